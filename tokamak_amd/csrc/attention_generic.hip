@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, GenericItems items, T* __restrict__ out, int nh, int nkv,
-    int hd, int vd, int ps, int max_pages, float scale, int span) {
+    int hd, int vd, int ps, int max_pages, float scale, int span, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) float q_s[QT][kMaxHd];
   __shared__ __attribute__((aligned(16))) float p_s[kWaves][kWave][QT];
   __shared__ long base_s[kWaves][kWave];  // where a key's values lie (a quad's, for tokens that run alone), or -1
@@ -278,6 +278,9 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
       float top = m_s[0];
 #pragma unroll
       for (int w = 1; w < kWaves; ++w) top = fmaxf(top, m_s[w]);
+      // a sink is one more term exp(sink) of the head's denominator: no key, no value, not scaled
+      const float sink = sinks ? sinks[HEADS ? head0 + t : head0] : -INFINITY;
+      top = fmaxf(top, sink);
       float sum = 0.f, o = 0.f;
 #pragma unroll
       for (int w = 0; w < kWaves; ++w) {
@@ -285,6 +288,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
         sum = fmaf(l_s[w], e, sum);
         o = fmaf(acc_s[w][tid], e, o);
       }
+      if (sinks) sum += expf(sink - top);
       Elem<T>::store(out + row[t] * vd + tid, o / sum);
     }
   }
@@ -294,13 +298,14 @@ template <typename T, int SLOTS>
 static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const int* block_tables,
                            const int* positions, const int* req_of_token, GenericItems items,
                            int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int vd, int ps,
-                           int max_pages, float scale, int span, int share_heads, hipStream_t stream) {
+                           int max_pages, float scale, int span, int share_heads, const float* sinks,
+                           hipStream_t stream) {
   const int group = nh / nkv;
 #define TK_ALONE(QT_)                                                                               \
   paged_attention_generic_kernel<T, QT_, true, SLOTS>                                               \
       <<<dim3(num_single, nkv, (group + QT_ - 1) / QT_), kWaves * kWave, 0, stream>>>(              \
           q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd,  \
-          ps, max_pages, scale, span)
+          ps, max_pages, scale, span, sinks)
   if (num_single > 0) {
     // the heads of a group share a block if that still gives every CU one (the result is the
     // same either way): at batch 64 of an 8B-shaped layer a third faster, at batch 8 slower
@@ -316,20 +321,21 @@ static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const
     paged_attention_generic_kernel<T, kQueries, false, SLOTS>
         <<<dim3(num_tiles, nh, kTileTokens / kQueries), kWaves * kWave, 0, stream>>>(
             q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd, ps,
-            max_pages, scale, span);
+            max_pages, scale, span, sinks);
 }
 
 // tile_first / tile_count (num_tiles of them) and single (num_single token rows): the step's work
 // lists, which together name every token once.  With tile_first null every one of the N tokens
 // runs alone.  share_heads: whether the query heads of a group share a block for the tokens
-// that run alone (1), or not (0), or as fills the GPU (-1); the result is the same.
+// that run alone (1), or not (0), or as fills the GPU (-1); the result is the same.  sinks: null, or
+// float32 [nh]: head a's softmax has exp(sinks[a]) as one more term of its denominator.
 TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_cache,
                                       const void* v_cache, const int* block_tables,
                                       const int* positions, const int* req_of_token, void* out,
                                       int N, int nh, int nkv, int hd, int vd, int ps, int max_pages,
                                       float scale, int span, const int* tile_first,
                                       const int* tile_count, int num_tiles, const int* single,
-                                      int num_single, int share_heads, hipStream_t stream) {
+                                      int num_single, int share_heads, const float* sinks, hipStream_t stream) {
   if (N <= 0) return 0;
   if (hd > kMaxHd || hd % 8 != 0 || vd > kMaxHd || vd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
   if (tile_first == nullptr) {
@@ -343,7 +349,7 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
 #define TK_GENERIC(T_, SLOTS_)                                                                      \
   launch_generic<T_, SLOTS_>((const T_*)q, (const T_*)k_cache, (const T_*)v_cache, block_tables,    \
                              positions, req_of_token, items, num_single, num_tiles, (T_*)out, nh,   \
-                             nkv, hd, vd, ps, max_pages, scale, span, share_heads, stream)
+                             nkv, hd, vd, ps, max_pages, scale, span, share_heads, sinks, stream)
   if (dtype == 0) {
     if (vd <= 128) TK_GENERIC(float, 2);
     else if (vd <= 256) TK_GENERIC(float, 4);

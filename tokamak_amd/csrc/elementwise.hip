@@ -237,23 +237,25 @@ TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, int delta_
 // rotary tables: angle = float(pos) * inv_freq[j]  (one float32 product, as the
 // formula is written), cos/sin [N, half]
 // ---------------------------------------------------------------------------
+// `amplitude` multiplies both tables (1: as they are).
 __global__ void rope_tables_kernel(const int* __restrict__ positions,
                                    const float* __restrict__ inv_freq, float* __restrict__ cos_t,
-                                   float* __restrict__ sin_t, int N, int half) {
+                                   float* __restrict__ sin_t, int N, int half, float amplitude) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= N * half) return;
   const int n = i / half, j = i - n * half;
   const float angle = __fmul_rn((float)positions[n], inv_freq[j]);
-  cos_t[i] = cosf(angle);
-  sin_t[i] = sinf(angle);
+  const float c = cosf(angle), s = sinf(angle);
+  cos_t[i] = amplitude == 1.f ? c : c * amplitude;
+  sin_t[i] = amplitude == 1.f ? s : s * amplitude;
 }
 
 TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* cos_t, float* sin_t,
-                          int N, int half, hipStream_t stream) {
+                          int N, int half, float amplitude, hipStream_t stream) {
   const int total = N * half;
   if (total <= 0) return 0;
   rope_tables_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, cos_t, sin_t, N,
-                                                               half);
+                                                               half, amplitude);
   return launch_status();
 }
 
@@ -534,22 +536,28 @@ TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int part
 }
 
 // ---------------------------------------------------------------------------
-// out[n, i] = silu(gu[n, i]) * gu[n, I + i],  silu(z) = z / (1 + exp(-z))
+// out[n, i] = act(gu[n, i]) * gu[n, I + i]; act 0: silu(z) = z / (1 + exp(-z)), act 1: the tanh
+// form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float gate_act(float z, int act) {
+  if (act == 0) return z / (1.f + expf(-z));
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, int act) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t n = idx / I;
   const int i = (int)(idx - n * I);
   const float g = Elem<T>::load(gu + n * 2 * I + i);
   const float u = Elem<T>::load(gu + n * 2 * I + I + i);
-  Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
+  Elem<T>::store(out + idx, gate_act(g, act) * u);
 }
 
 // 8 elements a thread (16-byte loads): I a multiple of 8, pointers 16-byte aligned
 __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
-                                       int I, size_t total8) {
+                                       int I, size_t total8, int act) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total8) return;
   const int per_row = I / 8;
@@ -563,25 +571,26 @@ __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __
   for (int k = 0; k < 4; ++k) {
     const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-    ow[k] = pack_bf16x2(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+    ow[k] = pack_bf16x2(gate_act(g0, act) * u0, gate_act(g1, act) * u1);
   }
   *reinterpret_cast<uint4*>(out + n * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, hipStream_t stream) {
+TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, int act, hipStream_t stream) {
   if (N <= 0 || I <= 0) return 0;
+  if (act != 0 && act != 1) return -1;
   const size_t total = (size_t)N * I;
   if (dtype == 1 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
     const size_t total8 = total / 8;
     silu_mul_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
-        (const bf16_t*)gu, (bf16_t*)out, I, total8);
+        (const bf16_t*)gu, (bf16_t*)out, I, total8, act);
     return launch_status();
   }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == 0)
-    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total, act);
   else
-    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total, act);
   return launch_status();
 }
 
@@ -670,7 +679,167 @@ TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long 
 }
 
 // ---------------------------------------------------------------------------
-// Half-split rotation of the first `rot` dims of q and k, THEN each head of q and k divided by
+// Residual add of two parallel branches + norm over rows of width H.
+//   x = resid[row] + (a[row] + b[row]);  if write_resid: resid[row] = x
+//   center: out[m] = (x - mean(x)) * rsqrt(mean((x - mean(x))^2) + eps) * weight   (a layer norm without a bias)
+//   else:   out[m] = x * rsqrt(mean(x^2) + eps) * weight
+// A branch is T, float32, or float32 partial sums (added in order); each may be absent.  The
+// two branches' sum is formed first, in float32, and added to the stream once.
+// ---------------------------------------------------------------------------
+struct NormBranch {
+  const void* p;
+  int f32;
+  int parts;
+  long stride;
+};
+
+template <typename T>
+__device__ __forceinline__ float4 branch_four(const NormBranch& b, size_t idx) {
+  if (!b.f32) return Load4<T>::at(reinterpret_cast<const T*>(b.p) + idx);
+  const float* f = reinterpret_cast<const float*>(b.p) + idx;
+  float4 s = *reinterpret_cast<const float4*>(f);
+  for (int i = 1; i < b.parts; ++i) {
+    const float4 q = *reinterpret_cast<const float4*>(f + (size_t)i * b.stride);
+    s.x += q.x; s.y += q.y; s.z += q.z; s.w += q.w;
+  }
+  return s;
+}
+
+template <typename T>
+__device__ __forceinline__ float branches_value(const NormBranch& a, const NormBranch& b, size_t idx) {
+  float s = 0.f;
+  if (a.p) s = branch_value<T>(a.p, a.f32, a.parts, a.stride, idx);
+  if (b.p) s += branch_value<T>(b.p, b.f32, b.parts, b.stride, idx);
+  return s;
+}
+
+// Vector form: a thread keeps up to kNormGroups pieces of four elements of the row in registers.
+template <typename T>
+__global__ __launch_bounds__(1024) void add_norm2_vec_kernel(
+    float* __restrict__ resid, NormBranch a, NormBranch b, const int* __restrict__ rows,
+    const float* __restrict__ weight, T* __restrict__ out, int H, float eps, int write_resid, int center) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const size_t row = rows ? (size_t)rows[m] : (size_t)m;
+  float* x = resid + row * H;
+  float4 xv[kNormGroups], wv[kNormGroups];
+  float sum = 0.f;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    wv[g] = d < H ? *reinterpret_cast<const float4*>(weight + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    xv[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d < H) {
+      float4 v = *reinterpret_cast<const float4*>(x + d);
+      if (a.p || b.p) {
+        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a.p) s = branch_four<T>(a, row * H + d);
+        if (b.p) {
+          const float4 t = branch_four<T>(b, row * H + d);
+          if (a.p) { s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w; }
+          else s = t;
+        }
+        v.x += s.x; v.y += s.y; v.z += s.z; v.w += s.w;
+        if (write_resid) *reinterpret_cast<float4*>(x + d) = v;
+      }
+      xv[g] = v;
+      sum += (v.x + v.y) + (v.z + v.w);
+    }
+  }
+  float mean = 0.f;
+  if (center) mean = block_sum(sum, scratch) / (float)H;
+  float ss = 0.f;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    if (d < H) {
+      xv[g].x -= mean; xv[g].y -= mean; xv[g].z -= mean; xv[g].w -= mean;
+      ss += xv[g].x * xv[g].x + xv[g].y * xv[g].y + xv[g].z * xv[g].z + xv[g].w * xv[g].w;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = 1.f / sqrtf(ss / (float)H + eps);
+  T* o = out + (size_t)m * H;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    if (d < H) {
+      const float4 w = wv[g];
+      Store4<T>::at(o + d, make_float4(xv[g].x * rstd * w.x, xv[g].y * rstd * w.y,
+                                       xv[g].z * rstd * w.z, xv[g].w * rstd * w.w));
+    }
+  }
+}
+
+// Any width and alignment: the row is walked three times (mean, variance, output).
+template <typename T>
+__global__ void add_norm2_kernel(float* __restrict__ resid, NormBranch a, NormBranch b,
+                                 const int* __restrict__ rows, const float* __restrict__ weight,
+                                 T* __restrict__ out, int H, float eps, int write_resid, int center) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const size_t row = rows ? (size_t)rows[m] : (size_t)m;
+  float* x = resid + row * H;
+  const bool adds = a.p || b.p;
+  float sum = 0.f;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) {
+    float v = x[d];
+    if (adds) {
+      v += branches_value<T>(a, b, row * H + d);
+      if (write_resid) x[d] = v;      // (the passes below then read the sum back)
+    }
+    sum += v;
+  }
+  const bool again = adds && !write_resid;    // the sum is not in the stream: it is formed again
+  float mean = 0.f;
+  if (center) mean = block_sum(sum, scratch) / (float)H;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) {
+    float v = x[d];
+    if (again) v += branches_value<T>(a, b, row * H + d);
+    ss += (v - mean) * (v - mean);
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = 1.f / sqrtf(ss / (float)H + eps);
+  T* o = out + (size_t)m * H;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) {
+    float v = x[d];
+    if (again) v += branches_value<T>(a, b, row * H + d);
+    Elem<T>::store(o + d, (v - mean) * rstd * weight[d]);
+  }
+}
+
+TK_API int tk_add_norm2(int dtype, float* resid, const void* a, int a_f32, int a_parts, long a_stride,
+                        const void* b, int b_f32, int b_parts, long b_stride, const int* rows,
+                        const float* weight, void* out, int M, int H, float eps, int write_resid,
+                        int center, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (rows && write_resid) return -1;
+  if (a_parts < 1 || b_parts < 1 || (a_parts > 1 && !a_f32) || (b_parts > 1 && !b_f32)) return -1;
+  const NormBranch ba{a, a_f32 || dtype == 0, a_parts, a_stride}, bb{b, b_f32 || dtype == 0, b_parts, b_stride};
+  int threads = 64;
+  while (threads < 1024 && threads * 4 * (M >= 512 ? kNormGroups : 1) < H) threads *= 2;
+  const bool vec = H % 4 == 0 && H <= threads * 4 * kNormGroups && a_stride % 4 == 0 && b_stride % 4 == 0 &&
+                   ((uintptr_t)resid % 16 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&
+                   ((uintptr_t)weight % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  if (vec) {
+    if (dtype == 0) add_norm2_vec_kernel<float><<<M, threads, 0, stream>>>(resid, ba, bb, rows, weight, (float*)out, H, eps, write_resid, center);
+    else add_norm2_vec_kernel<bf16_t><<<M, threads, 0, stream>>>(resid, ba, bb, rows, weight, (bf16_t*)out, H, eps, write_resid, center);
+  } else {
+    if (dtype == 0) add_norm2_kernel<float><<<M, 256, 0, stream>>>(resid, ba, bb, rows, weight, (float*)out, H, eps, write_resid, center);
+    else add_norm2_kernel<bf16_t><<<M, 256, 0, stream>>>(resid, ba, bb, rows, weight, (bf16_t*)out, H, eps, write_resid, center);
+  }
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// ---------------------------------------------------------------------------
+// Rotation of the first `rot` dims of q and k (half-split pairs, dim j with j + rot/2, or
+// `interleaved` pairs, dim 2j with 2j + 1), THEN (unit) each head of q and k divided by
 // its root mean square over all hd dims (times a weight per dim, if one is given), q written
 // out, k and v written into the paged cache.  Keys and values may differ in size:
 // qkv: [N, nh * hd + nkv_in * hd + nkv_in * vd] (q heads, k heads, v heads); with nkv_in == 0
@@ -679,6 +848,9 @@ TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long 
 // hdp >= hd and vdp >= vd are the sizes the pages and q_out are laid out for (hd rounded up to 8,
 // vd to 16): the channels behind hd are written as zeros into q_out and never written in the
 // pages (which start as zeros), so they add nothing to a score or an output.
+// Values may be mixed with those another layer made for the same tokens (v_keep, float32
+// [N, nkv * vd]): v_mode 1 leaves this layer's values there as they are projected; v_mode 2
+// caches (1 - lambda) v + lambda v_keep with lambda = *v_lambda.
 // One wave per (token, head), four waves a block, each with an LDS row of its own.
 // ---------------------------------------------------------------------------
 template <typename T, typename TIN>
@@ -688,7 +860,8 @@ __global__ void rope_norm_store_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
     T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int vd, int hdp, int vdp, int rot, int ps,
-    int max_pages, int unit, float eps, int num_pairs) {
+    int max_pages, int unit, float eps, int num_pairs, int interleaved, float* __restrict__ v_keep, int v_mode,
+    const float* __restrict__ v_lambda) {
   __shared__ float vecs[kPairsPerBlock][kMaxHeadDim];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int heads = nh + 2 * nkv_in;
@@ -714,15 +887,15 @@ __global__ void rope_norm_store_kernel(
     int cnt = 0;
     for (int j = lane; j < half; j += kWave, ++cnt) {
       const float c = cos_t[(size_t)n * half + j], s = sin_t[(size_t)n * half + j];
-      const float a = vec[j], b = vec[j + half];
+      const float a = vec[interleaved ? 2 * j : j], b = vec[interleaved ? 2 * j + 1 : j + half];
       lo[cnt] = a * c - b * s;
       hi[cnt] = b * c + a * s;
     }
     wave_lds_sync();
     cnt = 0;
     for (int j = lane; j < half; j += kWave, ++cnt) {
-      vec[j] = lo[cnt];
-      vec[j + half] = hi[cnt];
+      vec[interleaved ? 2 * j : j] = lo[cnt];
+      vec[interleaved ? 2 * j + 1 : j + half] = hi[cnt];
     }
     wave_lds_sync();
     if (unit) {
@@ -751,8 +924,14 @@ __global__ void rope_norm_store_kernel(
   } else {
     const int kvh = head - nh - nkv_in;
     T* base = v_cache + (size_t)page * ((size_t)nkv * vdp * ps) + (size_t)kvh * vdp * ps;
-    for (int d = lane; d < vd; d += kWave)
-      Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), vec[d]);
+    float* keep = v_keep + ((size_t)n * nkv + kvh) * vd;
+    const float lambda = v_mode == 2 ? *v_lambda : 0.f;
+    for (int d = lane; d < vd; d += kWave) {
+      float v = vec[d];
+      if (v_mode == 1) keep[d] = v;
+      else if (v_mode == 2) v = (1.f - lambda) * v + lambda * keep[d];
+      Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), v);
+    }
   }
 }
 
@@ -762,11 +941,13 @@ TK_API int tk_rope_norm_store(int dtype, const void* qkv, int in_f32, int parts,
                               const float* sin_t, const int* positions, const int* req_of_token,
                               const int* block_tables, void* q_out, void* k_cache, void* v_cache,
                               int N, int nh, int nkv_in, int nkv, int hd, int vd, int hdp, int vdp, int rot,
-                              int ps, int max_pages, int unit, float eps, hipStream_t stream) {
+                              int ps, int max_pages, int unit, float eps, int interleaved, float* v_keep,
+                              int v_mode, const float* v_lambda, hipStream_t stream) {
   if (N <= 0) return 0;
   if (hdp > kMaxHeadDim || vdp > kMaxHeadDim || hd < 1 || vd < 1 || hdp < hd || vdp < vd || hdp % 8 != 0 ||
       vdp % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0)
     return -1;
+  if (v_mode < 0 || v_mode > 2 || (v_mode != 0 && v_keep == nullptr) || (v_mode == 2 && v_lambda == nullptr)) return -1;
   if (nkv_in != 0 && nkv_in != nkv) return -1;
   if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
   const long pairs = (long)N * (nh + 2 * nkv_in);
@@ -776,7 +957,7 @@ TK_API int tk_rope_norm_store(int dtype, const void* qkv, int in_f32, int parts,
   rope_norm_store_kernel<T_, TIN_><<<grid, kWave * kPairsPerBlock, 0, stream>>>(                 \
       (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,         \
       req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, hd,   \
-      vd, hdp, vdp, rot, ps, max_pages, unit, eps, (int)pairs)
+      vd, hdp, vdp, rot, ps, max_pages, unit, eps, (int)pairs, interleaved, v_keep, v_mode, v_lambda)
   if (dtype == 0) TK_RN(float, float);
   else if (in_f32) TK_RN(bf16_t, float);
   else TK_RN(bf16_t, bf16_t);
@@ -803,6 +984,7 @@ TK_API int tk_scale_softcap(float* x, long total, float scale, float cap, hipStr
 
 // the same entry points in slot form (slots.h), for launch lists
 TK_SLOTS(tk_add_rmsnorm)
+TK_SLOTS(tk_add_norm2)
 TK_SLOTS(tk_rope_tables)
 TK_SLOTS(tk_qknorm_rope_store)
 TK_SLOTS(tk_silu_mul)

@@ -57,7 +57,7 @@ template <> struct Vec<bf16_t> {
 template <typename T>
 __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ chosen,
-    float* __restrict__ weight, int N, int W, int E, int top) {
+    float* __restrict__ weight, int N, int W, int E, int top, int softmax) {
   extern __shared__ float score[];     // [E]
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int n = blockIdx.x;
@@ -90,12 +90,23 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
     a0 = wave_sum(a0);
     a1 = wave_sum(a1);
     if (lane == 0) {
-      score[e] = 1.f / (1.f + expf(-a0));
-      if (e + 1 < E) score[e + 1] = 1.f / (1.f + expf(-a1));
+      score[e] = softmax ? a0 : 1.f / (1.f + expf(-a0));
+      if (e + 1 < E) score[e + 1] = softmax ? a1 : 1.f / (1.f + expf(-a1));
     }
   }
   __syncthreads();
   if (wave != 0) return;
+  if (softmax) {
+    // scores = softmax of the logits over all experts
+    float top_z = -INFINITY;
+    for (int e = lane; e < E; e += kWave) top_z = fmaxf(top_z, score[e]);
+    top_z = wave_max(top_z);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += kWave) sum += expf(score[e] - top_z);
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += kWave) score[e] = expf(score[e] - top_z) / sum;   // (a lane rewrites what it read)
+    wave_lds_sync();
+  }
   // the largest `top` scores, one after the other; a lane looks at the experts lane, lane + 64, ...
   for (int k = 0; k < top; ++k) {
     float best = -1.f;
@@ -131,7 +142,7 @@ __device__ __forceinline__ void load_piece(const T* p, float* o) {
 template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(
     const T* __restrict__ h, const T* __restrict__ gate_up, const int* __restrict__ chosen,
-    const float* __restrict__ weight, T* __restrict__ act, int W, int F, int top, int slab) {
+    const float* __restrict__ weight, T* __restrict__ act, int W, int F, int top, int slab, int on_output) {
   extern __shared__ float x[];         // [W]
   const int p = blockIdx.x, n = p / top;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
@@ -174,7 +185,9 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
 #pragma unroll
       for (int r = 0; r < kRows; ++r)
         if (r == lane) { gv = g[r]; uv = u[r]; }
-      gv *= wt;
+      // the weight on the expert's input scales both first products; on its output it scales
+      // the activations, which the second product carries through (it is linear)
+      if (!on_output) gv *= wt;
       uv *= wt;
       Elem<T>::store(act + (size_t)p * F + c0 + lane, gv / (1.f + expf(-gv)) * uv);
     }
@@ -303,7 +316,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ weights, const int* __restrict__ order,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_start, const int* __restrict__ tile_count,
     const int* __restrict__ num_tiles, const float* __restrict__ pair_weight, void* __restrict__ out,
-    int N, int top, int R, int K, int max_tiles, int channel_blocks) {
+    int N, int top, int R, int K, int max_tiles, int channel_blocks, int on_output) {
   int tile, channels;
   tile_of_block(max_tiles, channel_blocks, tile, channels);
   if (tile < 0 || tile >= *num_tiles) return;
@@ -392,7 +405,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
         float v[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float g = acc[i][j][q] * w, u = acc[NT + i][j][q] * w;
+          const float g = on_output ? acc[i][j][q] : acc[i][j][q] * w, u = acc[NT + i][j][q] * w;
           v[q] = g / (1.f + expf(-g)) * u;
         }
         bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)p * R + c;
@@ -418,7 +431,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ weights, const int* __restrict__ order,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_start, const int* __restrict__ tile_count,
     const int* __restrict__ num_tiles, const float* __restrict__ pair_weight, void* __restrict__ out,
-    int N, int top, int R, int K, int max_tiles, int channel_blocks) {
+    int N, int top, int R, int K, int max_tiles, int channel_blocks, int on_output) {
   int tile, channels;
   tile_of_block(max_tiles, channel_blocks, tile, channels);
   if (tile < 0 || tile >= *num_tiles) return;
@@ -513,7 +526,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         float v[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float g = acc[i][j][q] * w, u = acc[NT + i][j][q] * w;
+          const float g = on_output ? acc[i][j][q] : acc[i][j][q] * w, u = acc[NT + i][j][q] * w;
           v[q] = g / (1.f + expf(-g)) * u;
         }
         bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)p * R + c;
@@ -529,16 +542,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
 }  // namespace
 
 // h [N, W] in dtype; router [E, W] float32; chosen [N, top] int32 and weight [N, top] float32 out
+// softmax: the scores are the softmax of the logits over all experts, else their sigmoids
 TK_API int tk_moe_route(int dtype, const void* h, const float* router, int* chosen, float* weight, int N,
-                        int W, int E, int top, hipStream_t stream) {
+                        int W, int E, int top, int softmax, hipStream_t stream) {
   if (N <= 0) return 0;
   if (E < 1 || top < 1 || top > E || W < 1 || (size_t)E * 4 > 64 * 1024) return -1;
   const unsigned blocks = (unsigned)N;
   const size_t lds = (size_t)E * sizeof(float);
   if (dtype == 0)
-    moe_route_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>((const float*)h, router, chosen, weight, N, W, E, top);
+    moe_route_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>((const float*)h, router, chosen, weight, N, W, E, top, softmax);
   else
-    moe_route_kernel<bf16_t><<<blocks, kRouteWaves * kWave, lds, stream>>>((const bf16_t*)h, router, chosen, weight, N, W, E, top);
+    moe_route_kernel<bf16_t><<<blocks, kRouteWaves * kWave, lds, stream>>>((const bf16_t*)h, router, chosen, weight, N, W, E, top, softmax);
   return launch_status();
 }
 
@@ -551,8 +565,9 @@ static int slab_for(int channels, long rows) {
 }
 
 // act[N * top, F] = silu(w gate) * (w up) of every (token, chosen expert) pair
+// on_output: act = w * silu(gate) * up instead (the weight acts on the expert's output)
 TK_API int tk_moe_gate_up(int dtype, const void* h, const void* gate_up, const int* chosen, const float* weight,
-                          void* act, int N, int W, int F, int top, hipStream_t stream) {
+                          void* act, int N, int W, int F, int top, int on_output, hipStream_t stream) {
   if (N <= 0) return 0;
   const bool wide = W % (dtype == 0 ? 4 : 8) == 0;
   if ((size_t)W * 4 > 96 * 1024 || (long)N * top > 0x7fffffffL / 2) return -1;
@@ -569,7 +584,7 @@ TK_API int tk_moe_gate_up(int dtype, const void* h, const void* gate_up, const i
       allowed = true;                                                                                  \
     }                                                                                                  \
     moe_gate_up_kernel<T_, WIDE_><<<grid, 256, lds, stream>>>((const T_*)h, (const T_*)gate_up, chosen, weight, \
-                                                              (T_*)act, W, F, top, slab);              \
+                                                              (T_*)act, W, F, top, slab, on_output);   \
   }
   if (dtype == 0 && wide) TK_GU(float, true)
   else if (dtype == 0) TK_GU(float, false)
@@ -622,6 +637,8 @@ TK_API int tk_moe_sort(const int* chosen, int P, int E, int tile_pairs, int* ord
 }
 
 // bfloat16 only.  gated != 0: x [N][K] the tokens' rows, weights [E][2 R][K], out bfloat16 [N top][R];
+// gated == 2: as gated, but out = w * silu(g) * u (the pair's weight acts on the expert's output, which the
+// second product, being linear, carries through).
 // gated == 0: x [N top][K] the pairs' rows, weights [E][R][K], out float32 [top][N][R].
 // max_tiles: the length of the tile lists (blocks past num_tiles leave at once).
 TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const int* order, const int* tile_expert,
@@ -641,7 +658,7 @@ TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const i
   moe_grouped_wide_kernel<GATED_, ROWS_><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order, \
                                                                    tile_expert, tile_start, tile_count, num_tiles, \
                                                                    pair_weight, out, N, top, R, K, max_tiles,      \
-                                                                   channel_blocks)
+                                                                   channel_blocks, gated == 2)
     if (gated) TK_WIDE(true, 64);
     else TK_WIDE(false, 64);
 #undef TK_WIDE
@@ -653,12 +670,12 @@ TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const i
       moe_grouped_kernel<MT_, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,    \
                                                               tile_expert, tile_start, tile_count, num_tiles,     \
                                                               pair_weight, out, N, top, R, K, max_tiles,          \
-                                                              channel_blocks);                                    \
+                                                              channel_blocks, gated == 2);                        \
     else                                                                                                          \
       moe_grouped_kernel<MT_, false><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,   \
                                                                tile_expert, tile_start, tile_count, num_tiles,    \
                                                                pair_weight, out, N, top, R, K, max_tiles,         \
-                                                               channel_blocks);                                   \
+                                                               channel_blocks, 0);                                \
   }
   // rows_hint: the most pairs an expert can have (the step's pairs): tiles are never fuller than that
   if (rows_hint <= 16) TK_GROUPED(1)

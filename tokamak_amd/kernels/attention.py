@@ -273,7 +273,7 @@ def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, 
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads, num_kv_heads,
-                    head_dim, page_size, scale, window=None, value_dim=None, chunk=None) -> None:
+                    head_dim, page_size, scale, window=None, value_dim=None, chunk=None, sinks=None) -> None:
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages
     of each token's request.
 
@@ -288,6 +288,8 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     keys of its own chunk of that many positions only: the tiles of prompt portions on the
     matrix cores where the shape fits (tiles of 16, walking from the chunk's first stage),
     single tokens (which read a chunk at most) and everything else in the generic kernel.
+    ``sinks``: float32 [num_heads], one more term exp(sinks[a]) of head a's denominator; the generic
+    kernel has it.
     """
     value_dim = head_dim if value_dim is None else value_dim
     work = work_of(batch)
@@ -304,13 +306,13 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             tile_keys = sum(n + c % chunk for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
         kv_token_bytes = num_kv_heads * (head_dim + value_dim) * q.element_size()
         flops_per_pair = 2.0 * num_heads * (head_dim + value_dim)
-    if not chunk and value_dim == head_dim and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
+    if sinks is None and not chunk and value_dim == head_dim and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
         if _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, num_heads=num_heads,
                                  num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale,
                                  note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
             return
     tiles = (work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single)
-    if (chunk and work.num_tiles and value_dim == head_dim
+    if (sinks is None and chunk and work.num_tiles and value_dim == head_dim
             and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, None)):
         if profiling:
             ops._note(f"portions {work.num_tiles} tiles, chunks of {chunk}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
@@ -330,7 +332,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-        scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles)
+        scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, sinks=sinks)
 
 
 def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *, num_heads, num_kv_heads,

@@ -132,13 +132,20 @@ def _sink_fits(sink: StreamSink, m: int, n: int) -> bool:
             and (g is None or (g.dtype == torch.float32 and g.numel() == n and g.is_contiguous() and g.data_ptr() % 16 == 0)))
 
 
-def gated_linear(x: torch.Tensor | DeferredNorm, gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x @ gate^T) * (x @ up^T) for ``gate_up`` = [gate; up] ([2I, K]) -> [M, I].
+def gated_linear(x: torch.Tensor | DeferredNorm, gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """act(x @ gate^T) * (x @ up^T) for ``gate_up`` = [gate; up] ([2I, K]) -> [M, I].
 
-    bfloat16 with up to 64 rows: one fused weight-streaming kernel.  Otherwise
-    the product, then the SiLU-gate kernel.
+    bfloat16 with up to 64 rows and the SiLU gate: one fused weight-streaming kernel.  Otherwise
+    the product, then the gate kernel (``activation``: "silu" or "gelu_tanh").
     """
     m = x.shape[0]
+    if activation != "silu":
+        if isinstance(x, DeferredNorm):
+            x = x.materialize()
+        out = torch.empty((m, gate_up.shape[0] // 2), dtype=x.dtype, device=x.device)
+        if m:
+            ops.silu_mul(linear(x, gate_up), out, activation)
+        return out
     inter = gate_up.shape[0] // 2
     # A very small pair of matrices (0.6B-shaped: 13 MB) goes to the whole-K form, whose blocks of 16
     # columns let their waves split K, which the streaming kernel cannot do under the gate: in a

@@ -170,15 +170,18 @@ _SIGS = {
         "tk_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p,
                            c_void_p, c_int, c_int, c_float, c_int, c_void_p],
-        "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "tk_add_norm2": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p,
+                         c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_int, c_void_p],
+        "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "tk_qknorm_rope_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
         "tk_rope_norm_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                               c_int, c_void_p, c_int, c_void_p, c_void_p],
         "tk_scale_softcap": [c_void_p, c_long, c_float, c_float, c_void_p],
-        "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "tk_scaled_sum": [c_int, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float,
                           c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
@@ -213,8 +216,9 @@ _SIGS = {
                         c_float, c_float, c_float, c_void_p],
     },
     "moe": {
-        "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-        "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p],
         "tk_moe_down": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_moe_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "tk_moe_grouped": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -248,7 +252,15 @@ _SIGS = {
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p,
+                                       c_void_p],
+    },
+    "latent": {
+        "tk_latent_prepare": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+        "tk_head_linear": [c_int, c_void_p, c_long, c_long, c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int,
+                           c_int, c_void_p],
     },
     "attention_mfma": {
         "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -420,15 +432,41 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
                                                 int(bool(write_resid)), _stream()), "add_rmsnorm")
 
 
+def add_norm2(resid: torch.Tensor, a: torch.Tensor | None, b: torch.Tensor | None, weight: torch.Tensor, eps: float,
+              out: torch.Tensor, *, center: bool, rows: torch.Tensor | None = None, write_resid: bool = True) -> None:
+    """x = resid[row] + (a[row] + b[row]), optionally stored back; ``center``: out = (x - mean) /
+    sqrt(mean((x - mean)^2) + eps) * weight (a layer norm without a bias), else the RMS norm.  ``a`` and
+    ``b`` are each None, [M, H] in the compute dtype or float32, or float32 partial sums [P, M, H]."""
+    _gpu(resid, a, b, weight, out, rows)
+    h = resid.shape[-1]
+    m = out.shape[0] if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and weight.dtype == torch.float32, "residual and norm weight are float32")
+    _need(weight.numel() == h and out.shape[-1] == h and out.shape[0] >= m, "norm shapes disagree")
+    adds = a is not None or b is not None
+    if rows is None:
+        _need(resid.shape[0] >= m, "residual has fewer rows than the output")
+    else:
+        _need(rows.dtype == torch.int32 and not (write_resid and adds), "a row-indexed norm cannot write the residual")
+        write_resid = False
+    pa, fa, na, sa = _branch(a, resid.shape[0], h, out.dtype, "a")
+    pb, fb, nb, sb = _branch(b, resid.shape[0], h, out.dtype, "b")
+    _note(f"{m}x{h}", m * h * (4 + (8 if write_resid and adds else 0) + out.element_size())
+          + sum(t.element_size() * parts * m * h for t, parts in ((a, na), (b, nb)) if t is not None))
+    _check(_fn("elementwise", "tk_add_norm2")(_code(out.dtype), _p(resid), pa, fa, na, sa, pb, fb, nb, sb, _p(rows),
+                                              _p(weight), _p(out), m, h, float(eps), int(bool(write_resid)),
+                                              int(bool(center)), _stream()), "add_norm2")
+
+
 def rope_tables(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor,
-                sin: torch.Tensor) -> None:
+                sin: torch.Tensor, amplitude: float = 1.0) -> None:
+    """cos and sin of float(position) * inv_freq[j], float32 [N, half], both times ``amplitude``."""
     _gpu(positions, inv_freq, cos, sin)
     n, half = positions.numel(), inv_freq.numel()
     _need(positions.dtype == torch.int32 and inv_freq.dtype == torch.float32, "positions int32, inv_freq float32")
     _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.numel() >= n * half
           and sin.numel() >= n * half, "cos/sin tables must be float32 [N, half]")
     _check(_fn("elementwise", "tk_rope_tables")(_p(positions), _p(inv_freq), _p(cos), _p(sin), n,
-                                                half, _stream()), "rope_tables")
+                                                half, float(amplitude), _stream()), "rope_tables")
 
 
 def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
@@ -475,15 +513,29 @@ def rope_norm_store(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: 
                     req_of_token: torch.Tensor, block_tables: torch.Tensor, q_out: torch.Tensor,
                     k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, value_dim: int, rotary_dim: int, page_size: int, unit_norm: bool, eps: float,
-                    store: bool = True) -> None:
+                    store: bool = True, interleaved: bool = False, value_keep: torch.Tensor | None = None,
+                    value_mode: int = 0, value_lambda: torch.Tensor | None = None) -> None:
     """Rotation of the first ``rotary_dim`` dims of every q and k head, then (``unit_norm``) each
     head divided by its root mean square over ``head_dim`` (times a weight, if given); q written to
     q_out, k and v into pages.  Values are ``value_dim`` wide.  ``rotary_dim`` 0: no rotation.
     q_out and the pages are laid out for ``padded_sizes(head_dim, value_dim)``: the channels behind
-    the true sizes hold zeros."""
-    _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache)
+    the true sizes hold zeros.  ``interleaved``: the rotation pairs dim 2j with 2j + 1 instead of j with
+    j + rotary_dim / 2.  ``value_mode`` 1: the values, as projected, are also left in ``value_keep`` (float32
+    [N, kv heads * value_dim]); 2: what is cached is (1 - lambda) v + lambda value_keep with lambda =
+    ``value_lambda`` (one float32 number on the device)."""
+    _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache,
+         value_keep, value_lambda)
     n = positions.numel()
     nkv_in = num_kv_heads if store else 0
+    if not store:
+        value_mode = 0
+    _need(value_mode in (0, 1, 2), "value_mode is 0, 1 or 2")
+    if value_mode:
+        _need(value_keep is not None and value_keep.dtype == torch.float32
+              and value_keep.numel() >= n * num_kv_heads * value_dim, "the kept values are float32 [N, kv heads * value_dim]")
+    if value_mode == 2:
+        _need(value_lambda is not None and value_lambda.dtype == torch.float32 and value_lambda.numel() == 1,
+              "the mixing weight is one float32 number")
     width = (num_heads + nkv_in) * head_dim + nkv_in * value_dim
     in_f32, parts, stride = _partials(qkv, n, width, q_out.dtype, "qkv")
     hdp, vdp = padded_sizes(head_dim, value_dim)
@@ -510,7 +562,8 @@ def rope_norm_store(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: 
         _code(q_out.dtype), _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
         _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
         nkv_in, num_kv_heads, head_dim, value_dim, hdp, vdp, rotary_dim, page_size, block_tables.shape[1],
-        int(bool(unit_norm)), float(eps), _stream()), "rope_norm_store")
+        int(bool(unit_norm)), float(eps), int(bool(interleaved)), _p(value_keep if value_mode else None), int(value_mode),
+        _p(value_lambda if value_mode == 2 else None), _stream()), "rope_norm_store")
 
 
 def padded_sizes(head_dim: int, value_dim: int) -> tuple[int, int]:
@@ -527,14 +580,18 @@ def scale_softcap(logits: torch.Tensor, scale: float, cap: float | None) -> None
            "scale_softcap")
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """out[n, i] = act(gate_up[n, i]) * gate_up[n, I + i]; act is silu, or the tanh form of gelu."""
     _gpu(gate_up, out)
     n, two_i = gate_up.shape
     _need(two_i % 2 == 0 and out.shape == (n, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes disagree")
     _note(f"{n}x{two_i // 2}", n * two_i * out.element_size() * 1.5)
+    _need(activation in GATE_ACTIVATIONS, f"the gate's activation is one of {sorted(GATE_ACTIVATIONS)}")
     _check(_fn("elementwise", "tk_silu_mul")(_code(out.dtype), _p(gate_up), _p(out), n, two_i // 2,
-                                             _stream()), "silu_mul")
+                                             GATE_ACTIVATIONS[activation], _stream()), "silu_mul")
 
 
 def _branch(t: torch.Tensor | None, rows: int, width: int, dtype: torch.dtype, what: str):
@@ -837,23 +894,28 @@ def gla_column_splits(requests: int, heads: int, vdim: int, longest: int) -> int
 MOE_LDS_BYTES = 96 * 1024      # of a row of activations in float32 that a block of the expert kernels stages
 
 
-def moe_route(h: torch.Tensor, router: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, top: int) -> None:
-    """Per token the ``top`` experts with the largest sigmoid(router . h), float32 throughout:
+def moe_route(h: torch.Tensor, router: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, top: int,
+              scoring: str = "sigmoid") -> None:
+    """Per token the ``top`` experts with the largest scores, float32 throughout: the scores are
+    sigmoid(router . h), or with ``scoring="softmax"`` the softmax of router . h over all experts;
     chosen [N, top] int32 (largest first, the lower index on ties), weight [N, top] float32 their scores."""
+    _need(scoring in ("sigmoid", "softmax"), "the router's scores are sigmoids or a softmax")
     _gpu(h, router, chosen, weight)
     n, w = h.shape
     e = router.shape[0]
     _need(router.dtype == torch.float32 and router.shape == (e, w), "the router is float32 [experts, width]")
     _need(1 <= top <= e and chosen.dtype == torch.int32 and weight.dtype == torch.float32
           and chosen.numel() >= n * top and weight.numel() >= n * top, "lists of chosen experts too small")
-    _check(_fn("moe", "tk_moe_route")(_code(h.dtype), _p(h), _p(router), _p(chosen), _p(weight), n, w, e, top, _stream()),
-           "moe_route")
+    _check(_fn("moe", "tk_moe_route")(_code(h.dtype), _p(h), _p(router), _p(chosen), _p(weight), n, w, e, top,
+                                      int(scoring == "softmax"), _stream()), "moe_route")
 
 
 def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, act: torch.Tensor,
-                top: int) -> None:
+                top: int, weight_on_output: bool = False) -> None:
     """act[n * top + k] = silu(w gate_e h[n]) * (w up_e h[n]) for the token's k-th chosen expert e with
-    weight w; gate_up [experts, 2 ff, width] holds an expert's gate rows, then its up rows."""
+    weight w; gate_up [experts, 2 ff, width] holds an expert's gate rows, then its up rows.
+    ``weight_on_output``: w * silu(gate_e h[n]) * (up_e h[n]) instead, so that the second product, which
+    is linear, yields w times the expert's output."""
     _gpu(h, gate_up, chosen, weight, act)
     n, w = h.shape
     e, two_f, w2 = gate_up.shape
@@ -863,7 +925,7 @@ def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, we
     _need(w * 4 <= MOE_LDS_BYTES, "a row of activations must fit LDS")
     _note(f"{n}x{top} {two_f}x{w}", min(n * top, e) * two_f * w * h.element_size(), 2.0 * n * top * two_f * w)
     _check(_fn("moe", "tk_moe_gate_up")(_code(h.dtype), _p(h), _p(gate_up), _p(chosen), _p(weight), _p(act), n, w, f, top,
-                                        _stream()), "moe_gate_up")
+                                        int(bool(weight_on_output)), _stream()), "moe_gate_up")
 
 
 def moe_down(act: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, out: torch.Tensor, top: int) -> None:
@@ -910,10 +972,11 @@ def moe_sort(chosen: torch.Tensor, num_experts: int, tile_pairs: int = MOE_TILE_
 
 
 def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weight: torch.Tensor | None,
-                out: torch.Tensor, *, tokens: int, top: int, gated: bool) -> None:
+                out: torch.Tensor, *, tokens: int, top: int, gated: bool, weight_on_output: bool = False) -> None:
     """One of the experts' two products over the tiles of ``lists`` (``moe_sort``), bfloat16 on the matrix
     cores.  ``gated``: x [tokens, K] the tokens' rows, weights [E, 2 R, K] (gate rows, then up rows), out
-    bfloat16 [tokens * top, R] = silu(w g) * (w u) with the pairs' weights w.  Else: x [tokens * top, K] the
+    bfloat16 [tokens * top, R] = silu(w g) * (w u) with the pairs' weights w (``weight_on_output``:
+    w * silu(g) * u).  Else: x [tokens * top, K] the
     pairs' rows, weights [E, R, K], out float32 [top, tokens, R]."""
     order, tile_expert, tile_start, tile_count, num_tiles, tile_pairs = lists
     _gpu(x, weights, pair_weight, out)
@@ -929,7 +992,7 @@ def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weigh
         _need(out.dtype == torch.float32 and out.shape == (top, tokens, r), "the pairs' outputs are float32 [top, tokens, width]")
     _note(f"{tokens}x{top} {weights.shape[1]}x{k}", min(tokens * top, e) * weights.shape[1] * k * 2, 2.0 * tokens * top * weights.shape[1] * k)
     _check(_fn("moe", "tk_moe_grouped")(
-        int(gated), _p(x), _p(weights), _p(order), _p(tile_expert), _p(tile_start), _p(tile_count), _p(num_tiles),
+        (2 if weight_on_output else 1) if gated else 0, _p(x), _p(weights), _p(order), _p(tile_expert), _p(tile_start), _p(tile_count), _p(num_tiles),
         _p(pair_weight), _p(out), tokens, top, r, k, tile_expert.numel(), tokens * top, tile_pairs, _stream()), "moe_grouped")
 
 
@@ -1258,13 +1321,71 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tile
                                               w.stride(0), out.stride(0), row_tiles, waves, _stream()), "gemm_skinny")
 
 
+def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor | None, cos: torch.Tensor | None,
+                   sin: torch.Tensor | None, positions: torch.Tensor, req_of_token: torch.Tensor,
+                   block_tables: torch.Tensor, q_plain: torch.Tensor, q_full: torch.Tensor,
+                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int, head_dim: int,
+                   rot_dim: int, rank: int, rotary_dim: int, interleaved: bool, page_size: int, eps: float,
+                   store: bool = True) -> None:
+    """From a token's projections [q heads of (head_dim unrotated | rot_dim rotated) | latent of ``rank`` |
+    one key part of rot_dim] (the last two only with ``store``): the unrotated query parts to q_plain
+    [N, heads, head_dim]; the rotated ones into q_full[n, a, rank : rank + rot_dim] (q_full is [N, heads,
+    padded key size]; its first ``rank`` channels are left for the query carried into the latent's space);
+    the latent divided by its root mean square (``eps``) times ``latent_weight`` and the rotated key part
+    into the K page as one key [latent | rotated part], the latent also into the V page."""
+    _gpu(proj, latent_weight, cos, sin, positions, req_of_token, block_tables, q_plain, q_full, k_cache, v_cache)
+    n = positions.numel()
+    qw = head_dim + rot_dim
+    width = num_heads * qw + (rank + rot_dim if store else 0)
+    in_f32, parts, stride = _partials(proj, n, width, q_full.dtype, "projections")
+    hdp, vdp = padded_sizes(rank + rot_dim, rank)
+    _need(max(qw, rank + rot_dim) <= 1024 and max(hdp, vdp) <= 512, "heads of up to 1,024 and keys of up to 512 channels")
+    _need(q_plain.dtype == q_full.dtype and q_plain.numel() >= n * num_heads * head_dim
+          and q_full.numel() >= n * num_heads * hdp, "q_plain / q_full too small")
+    _need(rotary_dim % 2 == 0 and 0 <= rotary_dim <= rot_dim and page_size % 8 == 0, "rotary_dim is even and at most rot_dim")
+    _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32
+                               and sin.dtype == torch.float32 and cos.numel() >= n * (rotary_dim // 2)
+                               and sin.numel() >= n * (rotary_dim // 2)), "rotary tables missing, not float32 or too small")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and req_of_token.numel() >= n
+          and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    if store:
+        _need(latent_weight is not None and latent_weight.dtype == torch.float32 and latent_weight.numel() == rank,
+              "the latent's norm weight is float32 [rank]")
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_full.dtype == v_cache.dtype
+              and k_cache.numel() % (hdp * page_size) == 0 and v_cache.numel() % (vdp * page_size) == 0
+              and k_cache.numel() // hdp == v_cache.numel() // vdp, "cache size is not whole pages")
+    _note(f"{n}x{width}", n * width * (proj.element_size() * parts + q_full.element_size()))
+    _check(_fn("latent", "tk_latent_prepare")(
+        _code(q_full.dtype), _p(proj), in_f32, parts, stride, _p(latent_weight), _p(cos), _p(sin), _p(positions),
+        _p(req_of_token), _p(block_tables), _p(q_plain), _p(q_full), _p(k_cache if store else None),
+        _p(v_cache if store else None), n, num_heads, head_dim, rot_dim, rank, hdp, vdp, rotary_dim,
+        int(bool(interleaved)), page_size, block_tables.shape[1], float(eps), int(bool(store)), _stream()), "latent_prepare")
+
+
+def head_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n, a, :] = weight[a] @ x[n, a, :]: a product per head.  x [N, heads, K] and out [N, heads, M] may
+    be views with strides between rows and heads (the last dimension dense); weight [heads, M, K] is dense."""
+    _need(x.is_cuda and weight.is_cuda and out.is_cuda, "kernel arguments must live on the GPU (there is no CPU path)")
+    _need(x.dim() == 3 and out.dim() == 3 and weight.dim() == 3 and weight.is_contiguous(), "operands are [N, heads, K], [heads, M, K], [N, heads, M]")
+    n, heads, k = x.shape
+    m = weight.shape[1]
+    _need(weight.shape == (heads, m, k) and out.shape == (n, heads, m), "head_linear shapes disagree")
+    _need(x.dtype == weight.dtype == out.dtype and x.stride(2) == 1 and out.stride(2) == 1, "one dtype, dense last dimension")
+    if n == 0:
+        return
+    _note(f"{n}x{heads} {m}x{k}", (weight.numel() + x.numel() + out.numel()) * x.element_size(), 2.0 * n * heads * m * k)
+    _check(_fn("latent", "tk_head_linear")(_code(x.dtype), _p(x), x.stride(0), x.stride(1), _p(weight), _p(out),
+                                           out.stride(0), out.stride(1), n, heads, m, k, _stream()), "head_linear")
+
+
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_tables: torch.Tensor, positions: torch.Tensor,
                             req_of_token: torch.Tensor, out: torch.Tensor, *, num_heads: int,
                             num_kv_heads: int, head_dim: int, page_size: int, scale: float,
                             window: int | None = None, tiles: tuple | None = None,
                             share_heads: bool | None = None, value_dim: int | None = None,
-                            chunk: int | None = None, only_single: bool = False) -> None:
+                            chunk: int | None = None, only_single: bool = False,
+                            sinks: torch.Tensor | None = None) -> None:
     """Causal attention of each query token over its request's pages.  ``tiles``:
     (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
     of up to 16 consecutive tokens of one request, and token rows that run alone), which together
@@ -1274,8 +1395,10 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     how many there are; the same bits again.  ``value_dim``: size of a value head if it differs from
     ``head_dim``.  ``chunk``: a query sees only the keys of its own chunk of that many positions
     (counted from position 0); not together with ``window``.  ``only_single``: the tokens of the tiles
-    are left to another kernel."""
-    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
+    are left to another kernel.  ``sinks``: float32 [num_heads]; head a's softmax has exp(sinks[a]) as one
+    more term of its denominator, with no key and no value."""
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out, sinks)
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads), "sinks are float32 [num_heads]")
     n = positions.numel()
     vd = head_dim if value_dim is None else int(value_dim)
     _need(not (window and chunk), "a window or chunks, not both")
@@ -1310,7 +1433,8 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
         _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, vd, page_size,
         block_tables.shape[1], float(scale), span, _p(tile_first), _p(tile_count), num_tiles,
-        _p(single), num_single, -1 if share_heads is None else int(share_heads), _stream()), "paged_attention_generic")
+        _p(single), num_single, -1 if share_heads is None else int(share_heads), _p(sinks), _stream()),
+        "paged_attention_generic")
 
 
 NOT_INSTANTIATED = -2

@@ -138,15 +138,28 @@ class PositionData:
     """What a position encoding hands to a mixer for one step.
 
     ``cos``/``sin``: float32 [N, rotary_dim / 2] tables for a mixer that rotates
-    queries and keys (half-split pairing), or None.  ``score_slopes``: float32
+    queries and keys, or None; ``interleaved``: pair j is dimensions (2j, 2j + 1), else
+    (j, j + rotary_dim / 2).  ``score_slopes``: float32
     [heads] for a mixer that adds ``slope * (key position - query position)`` to its
     scores, or None.  A mixer refuses what it has no kernel for."""
 
     cos: torch.Tensor | None = None
     sin: torch.Tensor | None = None
     rotary_dim: int = 0
+    interleaved: bool = False
     score_slopes: torch.Tensor | None = None
     extra: dict = field(default_factory=dict)
+
+
+@dataclass
+class BranchPair:
+    """The outputs of two sub-layers that read the same normed input, not yet added to the residual
+    stream: each [N, H] in the compute dtype or float32, or float32 partial sums [P, N, H];
+    ``second`` may be None.  The norm that reads the stream next forms first + second in float32 and
+    adds the sum to the stream once."""
+
+    first: torch.Tensor
+    second: torch.Tensor | None = None
 
 
 class Embedding(Part):

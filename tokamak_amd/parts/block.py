@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels.linear import Added, StreamSink
-from tokamak_amd.parts.base import Block
+from tokamak_amd.parts.base import Block, BranchPair
 from tokamak_amd.parts.scale import scaled_sum
 
 
@@ -110,5 +110,35 @@ class ParallelMixersBlock(Block):
         return scaled_sum(out, 1.0, None, 0.0, self.feed_forward_scale.weight, dim, dtype)
 
 
+class ParallelSublayersBlock(Block):
+    """h = norm(x); x = x + (mixer(h) + feed_forward(h)).
+
+    One norm; the mixer and the feed-forward both read its output, and their outputs are added to
+    each other first and to the residual stream once, in float32, by the norm that reads the stream
+    next (it receives them as a ``BranchPair``).  The feed-forward may be absent: x = x + mixer(h).
+    An optional ``position`` part prepares the step's position data for the mixer.
+    """
+
+    roles = ("norm", "mixer")
+    optional = ("position", "feed_forward")
+    replays_parts = True
+
+    def __init__(self, parts) -> None:
+        super().__init__(parts)
+        self.norm = parts["norm"]
+        self.feed_forward = parts.get("feed_forward")
+        self.position = parts.get("position")
+        self.entry_norm = self.norm
+
+    def forward(self, resid, pending, batch, store, writes_cache):
+        position = None if self.position is None else self.position.prepare(batch)
+        h = self.norm.forward(resid, pending)
+        mixed = self.mixer.forward(h, batch, store, writes_cache, position)
+        if self.feed_forward is None:
+            return mixed
+        return BranchPair(mixed, self.feed_forward.forward(h, batch))
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel_sublayers", ParallelSublayersBlock)
 register_part("block", "parallel_mixers", ParallelMixersBlock)

@@ -14,12 +14,13 @@ class RoutedExperts(FeedForward):
     """``num_experts`` feed-forwards down(silu(gate x) * up x) without biases, of which every token
     uses ``top``.
 
-    The router's logits z = W_r h and the scores s = sigmoid(z) are float32; the ``top`` experts
+    The router's logits z = W_r h and the scores are float32: s = sigmoid(z), or with
+    ``scoring="softmax"`` the softmax of z over all experts; the ``top`` experts
     with the largest scores are chosen (the lower index on a tie) and weighted by their scores
     as they are, not renormalised.  ``weight_on`` says where a weight w acts: ``"input"``, the
     expert sees w * h (out = sum expert(w h)), or ``"output"``, out = sum w * expert(h).  On the
     input the kernels use gate(w h) = w gate(h): the weight scales the two first products in
-    float32.  Tensors: router, e<i>.gate, e<i>.up, e<i>.down; an expert's gate and up are held as
+    float32; on the output they use w down(a) = down(w a): the weight scales the activations.  Tensors: router, e<i>.gate, e<i>.up, e<i>.down; an expert's gate and up are held as
     one matrix and the experts as one array each.
     """
 
@@ -27,16 +28,18 @@ class RoutedExperts(FeedForward):
     replayable = True
 
     def __init__(self, *, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
-                 weight_on: str = "input", dtype, device,
+                 weight_on: str = "input", scoring: str = "sigmoid", dtype, device,
                  names: tuple[str, str, str, str, str] = ("router", "e{}.", "gate", "up", "down")) -> None:
         super().__init__(dtype=dtype, device=device)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.num_experts, self.top = int(num_experts), int(top)
         if not 1 <= self.top <= self.num_experts:
             raise ValueError(f"top ({top}) must be between 1 and the number of experts ({num_experts})")
-        if weight_on != "input":
-            raise ValueError(f"the expert kernels weigh an expert's input; weight_on={weight_on!r} has no kernel")
-        self.weight_on = weight_on
+        if weight_on not in ("input", "output"):
+            raise ValueError(f"weight_on is 'input' or 'output', got {weight_on!r}")
+        if scoring not in ("sigmoid", "softmax"):
+            raise ValueError(f"scoring is 'sigmoid' or 'softmax', got {scoring!r}")
+        self.weight_on, self.scoring = weight_on, scoring
         self.names = tuple(names)
         self.router = self.gate_up = self.down = None
 
@@ -68,16 +71,17 @@ class RoutedExperts(FeedForward):
         n, top = h.shape[0], self.top
         chosen = torch.empty((n, top), dtype=torch.int32, device=h.device)
         weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
-        ops.moe_route(h, self.router, chosen, weight, top)
+        ops.moe_route(h, self.router, chosen, weight, top, self.scoring)
+        on_output = self.weight_on == "output"
         act = torch.empty((n * top, self.intermediate_size), dtype=h.dtype, device=h.device)
         out = torch.empty((top, n, self.hidden_size), dtype=torch.float32, device=h.device)
         if ops.moe_grouped_fits(h, self.gate_up, self.down, n * top):
             # many tokens: the pairs listed expert by expert, tiles of one expert on the matrix cores
             lists = ops.moe_sort(chosen, self.num_experts)
-            ops.moe_grouped(h, self.gate_up, lists, weight, act, tokens=n, top=top, gated=True)
+            ops.moe_grouped(h, self.gate_up, lists, weight, act, tokens=n, top=top, gated=True, weight_on_output=on_output)
             ops.moe_grouped(act, self.down, lists, None, out, tokens=n, top=top, gated=False)
             return out
-        ops.moe_gate_up(h, self.gate_up, chosen, weight, act, top)
+        ops.moe_gate_up(h, self.gate_up, chosen, weight, act, top, on_output)
         ops.moe_down(act, self.down, chosen, out, top)
         return out
 
