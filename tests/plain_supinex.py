@@ -106,13 +106,15 @@ def attention(h, w, prefix, m, first_position=0, past=None, v_first=None):
     if past is not None:
         k, v = torch.cat([past[0], k]), torch.cat([past[1], v])
     group = heads // kv
+    size = int(m["mask"]["size"]) if m.get("mask") else None       # (a window, should a layer of this kind have one)
     out = torch.zeros(t, heads, vdim, dtype=h.dtype)
     for a in range(t):
         i = first_position + a
+        seen = [j for j in range(i + 1) if window_visible(i, j, size)]
         for head in range(heads):
-            scores = (k[: i + 1, head // group] @ q[a, head]) * float(m["scale"])
+            scores = (k[seen, head // group] @ q[a, head]) * float(m["scale"])
             p = sink_softmax(scores, w[prefix + "sink"][head] if prefix + "sink" in w else None)
-            out[a, head] = p @ v[: i + 1, head // group]
+            out[a, head] = p @ v[seen, head // group]
     return out.reshape(t, heads * vdim) @ w[prefix + "o"].T, (k, v), v_own
 
 

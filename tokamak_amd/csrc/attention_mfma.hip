@@ -130,7 +130,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
-    int split_keys, int nh, int nkv, int ps, float scale_log2, DecodeInputs in) {
+    int split_keys, int nh, int nkv, int ps, float scale_log2, DecodeInputs in, const float* __restrict__ sinks) {
   const bf16_t* __restrict__ k_cache = k_cache_in;
   const bf16_t* __restrict__ v_cache = v_cache_in;
   constexpr int KCH = HD / 32;  // 32-wide chunks of the head dim (QK^T steps)
@@ -367,6 +367,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
   const size_t row = (size_t)n0 * nh + kvh * G + head;
   const size_t prow = ((size_t)item * nh + kvh * G + head) * nsplit + split;  // partials are indexed by item, not token
   if (nsplit == 1) {
+    // a sink is one more term of the head's denominator (the maximum and the sums are in powers of two)
+    if (sinks) l_all += fast_exp2(sinks[kvh * G + head] * 1.4426950408889634f - m_all);
     const float inv = 1.f / l_all;
     *reinterpret_cast<uint2*>(out + row * HD + dim) =
         make_uint2(pack_bf16x2(o.x * inv, o.y * inv), pack_bf16x2(o.z * inv, o.w * inv));
@@ -388,7 +390,8 @@ template <int HD>
 __global__ __launch_bounds__(64) void attention_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     const int* __restrict__ positions, const int* __restrict__ item_token,
-    const int* __restrict__ item_count, bf16_t* __restrict__ out, int nsplit, int split_keys, int nh) {
+    const int* __restrict__ item_count, bf16_t* __restrict__ out, int nsplit, int split_keys, int nh,
+    const float* __restrict__ sinks) {
   const int head = blockIdx.y, lane = threadIdx.x;
   int n;
   if (item_count == nullptr) {
@@ -453,7 +456,9 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
       for (int i = 0; i < HD / 64; ++i) o[i] = fmaf(w, po[(size_t)t * HD + lane + i * 64], o[i]);
     }
   }
-  const float inv = 1.f / wave_sum(denom);
+  float denom_all = wave_sum(denom);
+  if (sinks) denom_all += fast_exp2(sinks[head] * 1.4426950408889634f - mx);
+  const float inv = 1.f / denom_all;
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) out[orow * HD + lane + i * 64] = float_to_bf16(o[i] * inv);
 }
@@ -487,7 +492,8 @@ void attention_prefill_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
-    int split_keys, int num_items, int nh, int nkv, int ps, float scale_log2, int chunk) {
+    int split_keys, int num_items, int nh, int nkv, int ps, float scale_log2, int chunk,
+    const float* __restrict__ sinks) {
   constexpr int KCH = HD / 32, DBL = HD / 16;
   constexpr int THREADS = kPrefillThreads;
   constexpr int GROUP_PIECES = 2 * HD;         // 16-byte pieces of K (and of V) per 16-key group
@@ -702,6 +708,7 @@ void attention_prefill_kernel(
   l += __shfl_xor(l, 32, kWave);
   if (c_valid && computes) {
     if (nsplit == 1) {
+      if (sinks) l += fast_exp2(sinks[head] * 1.4426950408889634f - m_run);
       const float inv = 1.f / l;
       bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + kb * 4;
 #pragma unroll
@@ -751,7 +758,8 @@ void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
-    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2,
+    const float* __restrict__ sinks) {
   constexpr int KST = HD / 16;  // 16-wide steps over the head dim (QK^T)
   constexpr int DB = HD / 32;   // 32-wide blocks of the head dim (PV outputs)
   constexpr int DBL = HD / 16;  // 16-dim blocks of a V page
@@ -929,6 +937,7 @@ void attention_prefill_wide_kernel(
   float l = l_run;
   l += __shfl_xor(l, 32, kWave);
   if (c_valid && computes) {
+    if (sinks) l += fast_exp2(sinks[head] * 1.4426950408889634f - m_run);
     const float inv = 1.f / l;
     bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + g * 4;
 #pragma unroll
@@ -966,7 +975,8 @@ void attention_prefill_group_kernel(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
-    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2,
+    const float* __restrict__ sinks) {
   constexpr int KST = HD / 16;  // 16-wide steps over the head dim (QK^T)
   constexpr int DB = HD / 32;   // 32-wide blocks of the head dim (PV outputs)
   constexpr int DBL = HD / 16;  // 16-dim blocks of a V page
@@ -1258,6 +1268,7 @@ void attention_prefill_group_kernel(
   float l = l_run;
   l += __shfl_xor(l, 32, kWave);
   if (c_valid && computes) {
+    if (sinks) l += fast_exp2(sinks[head] * 1.4426950408889634f - m_run);
     const float inv = 1.f / l;
     bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + g * 4;
 #pragma unroll
@@ -1278,17 +1289,18 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
                           const int* block_tables, int max_pages, const int* positions,
                           const int* req_of_token, const int* item_token, const int* item_count,
                           int num_items, void* out, float* part_o, float* part_ml, int nsplit,
-                          int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream, int chunk) {
+                          int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream, int chunk,
+                          const float* sinks) {
   const int G = nh / nkv;
   dim3 grid(nkv * (G / HPB), num_items, nsplit);
   attention_prefill_kernel<HD, HPB, OCC><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
-      split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f, chunk);
+      split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f, chunk, sinks);
   if (nsplit > 1) {
     dim3 mgrid(num_items * 16, nh);
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, item_count,
-                                                         (bf16_t*)out, nsplit, split_keys, nh);
+                                                         (bf16_t*)out, nsplit, split_keys, nh, sinks);
   }
   return launch_status();
 }
@@ -1298,13 +1310,13 @@ static int launch_prefill_wide(const void* q, const void* k_cache, const void* v
                                const int* block_tables, int max_pages, const int* positions,
                                const int* req_of_token, const int* item_token, const int* item_count,
                                int num_items, void* out, int nh, int nkv, int ps, float scale,
-                               hipStream_t stream) {
+                               hipStream_t stream, const float* sinks) {
   const int G = nh / nkv;
   dim3 grid(nkv * (G / HPB), num_items);
   attention_prefill_wide_kernel<HD, HPB><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
-      scale * 1.4426950408889634f);
+      scale * 1.4426950408889634f, sinks);
   return launch_status();
 }
 
@@ -1313,7 +1325,7 @@ static int launch_prefill_group(const void* q, const void* k_cache, const void* 
                                 const int* block_tables, int max_pages, const int* positions,
                                 const int* req_of_token, const int* item_token, const int* item_count,
                                 int num_items, void* out, int nh, int nkv, int ps, float scale,
-                                hipStream_t stream) {
+                                hipStream_t stream, const float* sinks) {
   const int G = nh / nkv;
   constexpr size_t one_stage = (size_t)S * 8 * HD * 16 * 2;                       // K and V of a stage
   constexpr size_t stage_bytes = 2 * one_stage <= 160 * 1024 ? 2 * one_stage : one_stage;  // two where they fit
@@ -1335,7 +1347,7 @@ static int launch_prefill_group(const void* q, const void* k_cache, const void* 
   attention_prefill_group_kernel<HD, GB, S><<<grid, GB * S * 64, lds, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
-      scale * 1.4426950408889634f);
+      scale * 1.4426950408889634f, sinks);
   return launch_status();
 }
 
@@ -1347,10 +1359,10 @@ static int launch_prefill_group_any(const void* q, const void* k_cache, const vo
                                     const int* block_tables, int max_pages, const int* positions,
                                     const int* req_of_token, const int* item_token, const int* item_count,
                                     int num_items, void* out, int nh, int nkv, int ps, float scale,
-                                    hipStream_t stream) {
+                                    hipStream_t stream, const float* sinks) {
 #define TK_GARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, nh, nkv, ps, scale, stream
+      num_items, out, nh, nkv, ps, scale, stream, sinks
   const int G = nh / nkv;
   const int nblk = (G + 7) / 8;
   const int gb = (G + nblk - 1) / nblk;  // heads a block: G itself up to 8, else an even share
@@ -1373,7 +1385,7 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
                   int max_pages, const int* positions, const int* req_of_token,
                   const int* item_token, const int* item_count, int num_items, void* out,
                   float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
-                  float scale, hipStream_t stream, DecodeInputs in = DecodeInputs{}) {
+                  float scale, hipStream_t stream, const float* sinks, DecodeInputs in = DecodeInputs{}) {
   if (num_items > 65535) return -1;
   dim3 grid(nkv, num_items, nsplit);
   const int G = nh / nkv;
@@ -1395,11 +1407,11 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
   attention_decode_kernel<HD, kDecodeWaves, 1, FUSED><<<grid, kDecodeWaves * 64, lds, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,
       req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps,
-      scale * 1.4426950408889634f, in);
+      scale * 1.4426950408889634f, in, sinks);
   if (nsplit > 1) {
     dim3 mgrid(num_items, nh);
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, nullptr,
-                                                         (bf16_t*)out, nsplit, split_keys, nh);
+                                                         (bf16_t*)out, nsplit, split_keys, nh, sinks);
   }
   return launch_status();
 }
@@ -1413,6 +1425,9 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
 // mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)
 // mode 3: tokens, wide form (item = up to 32 consecutive tokens of one request; nsplit must be 1)
 // mode 4: tokens, group form (items as in mode 3; any group size; a block holds a CU)
+// sinks: null, or float32 [nh]: head a's softmax has exp(sinks[a]) as one more term of its denominator
+// (no key, no value, not scaled); it is added where a row's sums are complete (the kernel's end, or
+// the merge of its splits).
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
 TK_API int tk_attention_decode_waves() { return kDecodeWaves; }
 
@@ -1421,7 +1436,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              const int* req_of_token, const int* item_token, const int* item_count,
                              int num_items, void* out, float* part_o, float* part_ml, int nsplit,
                              int split_keys, int nh, int nkv, int hd, int ps, float scale, int chunk,
-                             hipStream_t stream) {
+                             const float* sinks, hipStream_t stream) {
   if (num_items <= 0) return 0;
   if (mode < 0 || mode > 4) return -1;
   // chunked visibility: the narrow form for tiles only, their keys not split over blocks
@@ -1431,7 +1446,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
   const int G = nh / nkv;
 #define TK_ARGS                                                                                   \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, sinks
   if (mode == 0) {
     if (G > 16) return -2;
     if (hd == 128) return launch<128, false>(TK_ARGS);
@@ -1442,10 +1457,10 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     if (nsplit != 1) return -1;
     if (hd == 128) return launch_prefill_group_any<128>(q, k_cache, v_cache, block_tables, max_pages, positions,
                                                         req_of_token, item_token, item_count, num_items, out, nh,
-                                                        nkv, ps, scale, stream);
+                                                        nkv, ps, scale, stream, sinks);
     if (hd == 64) return launch_prefill_group_any<64>(q, k_cache, v_cache, block_tables, max_pages, positions,
                                                       req_of_token, item_token, item_count, num_items, out, nh,
-                                                      nkv, ps, scale, stream);
+                                                      nkv, ps, scale, stream, sinks);
     return -2;
   }
   const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
@@ -1453,7 +1468,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     if (nsplit != 1) return -1;
 #define TK_WARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, nh, nkv, ps, scale, stream
+      num_items, out, nh, nkv, ps, scale, stream, sinks
     // (groups of three heads and more take the group form; blocks of two heads or one here)
     if (hd == 128) {
       if (G % 2 == 0) return launch_prefill_wide<128, 2>(TK_WARGS);
@@ -1470,7 +1485,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
   if (nsplit > 1 && (split_keys % 64 != 0 || (long)num_items * 16 > 65535)) return -1;
 #define TK_PARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, chunk
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, chunk, sinks
   const bool dense = mode == 2;
   if (hd == 128) {
     if (hpb == 4) return dense ? launch_prefill<128, 4, 4>(TK_PARGS) : launch_prefill<128, 4, 2>(TK_PARGS);
@@ -1513,7 +1528,7 @@ TK_API int tk_attention_decode_fused(const void* qkv, int in_f32, int parts, lon
   DecodeInputs in{qkv, in_f32, parts, part_stride, q_weight, k_weight, cos_t, sin_t, rot, nkv_in, eps};
 #define TK_FARGS                                                                                       \
   nullptr, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, nullptr,  \
-      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, in
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, nullptr, in
   if (hd == 128) return launch<128, true>(TK_FARGS);
   if (hd == 64) return launch<64, true>(TK_FARGS);
 #undef TK_FARGS

@@ -288,8 +288,8 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     keys of its own chunk of that many positions only: the tiles of prompt portions on the
     matrix cores where the shape fits (tiles of 16, walking from the chunk's first stage),
     single tokens (which read a chunk at most) and everything else in the generic kernel.
-    ``sinks``: float32 [num_heads], one more term exp(sinks[a]) of head a's denominator; the generic
-    kernel has it.
+    ``sinks``: float32 [num_heads], one more term exp(sinks[a]) of head a's denominator, added where
+    a row's sums are complete (every kernel has it).
     """
     value_dim = head_dim if value_dim is None else value_dim
     work = work_of(batch)
@@ -306,25 +306,26 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             tile_keys = sum(n + c % chunk for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
         kv_token_bytes = num_kv_heads * (head_dim + value_dim) * q.element_size()
         flops_per_pair = 2.0 * num_heads * (head_dim + value_dim)
-    if sinks is None and not chunk and value_dim == head_dim and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
+    if not chunk and value_dim == head_dim and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
         if _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, num_heads=num_heads,
                                  num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale,
-                                 note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
+                                 sinks=sinks, note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
             return
     tiles = (work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single)
-    if (sinks is None and chunk and work.num_tiles and value_dim == head_dim
+    if (chunk and work.num_tiles and value_dim == head_dim
             and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, None)):
         if profiling:
             ops._note(f"portions {work.num_tiles} tiles, chunks of {chunk}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
         if ops.attention_mfma("tokens", q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token,
                               work.tile_first, work.tile_count, work.num_tiles, out, num_heads=num_heads,
-                              num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale, chunk=chunk):
+                              num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale, chunk=chunk,
+                              sinks=sinks):
             if profiling and work.num_single:
                 ops._note(f"{work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
             ops.paged_attention_generic(
                 q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
                 num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-                scale=scale, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True)
+                scale=scale, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
             return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
@@ -336,12 +337,12 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
 
 
 def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *, num_heads, num_kv_heads,
-                          head_dim, page_size, scale, note) -> bool:
+                          head_dim, page_size, scale, note, sinks=None) -> bool:
     """The matrix-core kernels over the step's single tokens and tiles.  False if the
     library has no instance for the shape: nothing of ``out`` counts then, and the caller
     runs the generic kernel over the whole step."""
     common = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
-                  page_size=page_size, scale=scale)
+                  page_size=page_size, scale=scale, sinks=sinks)
     if note is not None:
         decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair = note
     if work.num_single:

@@ -265,7 +265,7 @@ _SIGS = {
     "attention_mfma": {
         "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                              c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                              c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     },
     "attention_fused": {
         "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -1445,7 +1445,7 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                    item_token: torch.Tensor, item_count: torch.Tensor | None, num_items: int,
                    out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
                    page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1,
-                   chunk: int | None = None) -> bool:
+                   chunk: int | None = None, sinks: torch.Tensor | None = None) -> bool:
     """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
     decode token; "tokens": every item is up to 16 consecutive tokens of one
     request ("tokens_dense": the same, with the kernel variant for tiles that all
@@ -1455,9 +1455,11 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
     second kernel merges the pieces (in "heads" mode the sixteen waves of a block share a piece, so
     ``split_keys`` is a multiple of 256).  ``chunk`` ("tokens" and "tokens_dense" without splits): a
-    query sees the keys of its own chunk of that many positions only.  Returns False (nothing
+    query sees the keys of its own chunk of that many positions only.  ``sinks``: float32
+    [num_heads], one more term exp(sinks[a]) of head a's denominator.  Returns False (nothing
     launched) if the shape is not instantiated."""
-    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out)
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out, sinks)
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads), "sinks are float32 [num_heads]")
     n = positions.numel()
     _need(q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
           and out.dtype == torch.bfloat16, "the MFMA attention kernel takes bfloat16")
@@ -1489,7 +1491,7 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
         {"heads": 0, "tokens": 1, "tokens_dense": 2, "tokens_wide": 3, "tokens_group": 4}[mode], _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
         block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
         num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
-        head_dim, page_size, float(scale), int(chunk or 0), _stream())
+        head_dim, page_size, float(scale), int(chunk or 0), _p(sinks), _stream())
     if status == NOT_INSTANTIATED:
         return False
     _check(status, "attention_mfma")
