@@ -13,7 +13,8 @@
 //     K page [1][hdp/8][ps][8] receives [c | rotated part], V page [1][vdp/16][ps/4][16][4] receives c.
 //   head_linear: out[n, a, m] = sum_k x[n, a, k] W[a, m, k], a product per head, with row and head
 //     strides on both sides (q_plain -> q_full[.., :rank] with W = W_uk^T per head; the attention's
-//     output -> values with W = W_uv per head).  float32 accumulation over k ascending.
+//     output -> values with W = W_uv per head).  float32 accumulation over k ascending; bfloat16
+//     operands whose rows fill 16-byte pieces run on the matrix cores.
 #include "common.h"
 #include "slots.h"
 
@@ -136,6 +137,56 @@ __global__ __launch_bounds__(256) void head_linear_kernel(
   }
 }
 
+// bfloat16 on the matrix cores: a wave owns 16 output columns of one head for NT tiles of 16 tokens;
+// D^T[column][token] = W[column][:] . x[token][:] with v_mfma_f32_16x16x32_bf16, W rows as the A operand
+// (lane (row, kb) holds k = 32 c + 8 kb .. + 8) and x rows as B, both as 16-byte pieces straight from
+// memory (K a multiple of 8, rows 16-byte aligned); a lane ends with four consecutive columns of one
+// token.  float32 accumulation over k ascending in chunks of 32.
+typedef __bf16 hl_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hl_float4 __attribute__((ext_vector_type(4)));
+union HlFrag {
+  uint4 u;
+  hl_bf16x8 v;
+};
+
+template <int NT>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(
+    const bf16_t* __restrict__ x, long x_row, long x_head, const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+    long out_row, long out_head, int N, int M, int K) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
+  const int head = blockIdx.z;
+  const int m0 = (blockIdx.x * 4 + wave) * 16;
+  const int n0 = blockIdx.y * 16 * NT;
+  if (m0 >= M) return;   // (no barrier below)
+  const int wrow = min(m0 + col, M - 1);
+  const bf16_t* wp = w + ((size_t)head * M + wrow) * K + kb * 8;
+  const bf16_t* xp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+    xp[t] = x + (size_t)min(n0 + t * 16 + col, N - 1) * x_row + (size_t)head * x_head + kb * 8;
+  hl_float4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = hl_float4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool there = k0 + kb * 8 < K;   // (K is a multiple of 8: a piece is whole or absent)
+    HlFrag a, b[NT];
+    a.u = there ? *reinterpret_cast<const uint4*>(wp + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) b[t].u = there ? *reinterpret_cast<const uint4*>(xp[t] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[t].v, acc[t], 0, 0, 0);
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = n0 + t * 16 + col;
+    if (n >= N) continue;
+    bf16_t* op = out + (size_t)n * out_row + (size_t)head * out_head + m0 + kb * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (m0 + kb * 4 + e < M) op[e] = float_to_bf16(acc[t][e]);
+  }
+}
+
 }  // namespace
 
 // proj: [N, nh (dim + rot_dim) (+ rank + rot_dim if stores)] in dtype, or float32 (in_f32; possibly `parts`
@@ -173,6 +224,19 @@ TK_API int tk_head_linear(int dtype, const void* x, long x_row, long x_head, con
                           long out_row, long out_head, int N, int heads, int M, int K, hipStream_t stream) {
   if (N <= 0) return 0;
   if (heads < 1 || heads > 65535 || M < 1 || K < 1) return -1;
+  if (dtype != 0 && K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) {
+    // (tokens in tiles of 16: four tiles a wave once there are enough of them to fill the GPU without)
+    const int nt = (long)((N + 63) / 64) * ((M + 63) / 64) * heads >= 512 ? 4 : 1;
+    const dim3 mgrid((M + 63) / 64, (N + 16 * nt - 1) / (16 * nt), heads);
+    if (mgrid.y > 65535) return -1;
+    if (nt == 4)
+      head_linear_mfma_kernel<4><<<mgrid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w,
+                                                             (bf16_t*)out, out_row, out_head, N, M, K);
+    else
+      head_linear_mfma_kernel<1><<<mgrid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w,
+                                                             (bf16_t*)out, out_row, out_head, N, M, K);
+    return launch_status();
+  }
   const dim3 grid((M + kHlCols - 1) / kHlCols, (N + kHlRows - 1) / kHlRows, heads);
   if (grid.y > 65535) return -1;
   if (dtype == 0)

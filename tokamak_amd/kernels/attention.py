@@ -27,6 +27,8 @@ WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles 
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
 GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays
 GROUP_FILL = 128                # ... if its blocks times their shares of the keys are at least this many (half the CUs)
+TILES_ON_MATRIX_CORES = True    # bfloat16 portions that the tuned kernels do not take: csrc/attention_tiles.hip rather than
+                                # the generic kernel (tests of the generic kernel's own tiles switch this off)
 
 
 def quarter_octave_at_least(n: int, floor: int) -> int:
@@ -326,6 +328,25 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
                 q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
                 num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
                 scale=scale, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
+            return
+    if TILES_ON_MATRIX_CORES and work.num_tiles and q.dtype == torch.bfloat16 and page_size % 16 == 0:
+        # bfloat16 portions at shapes the tuned kernels do not take (unlike key and value sizes, other head
+        # sizes, a window): tiles of 16 tokens on the matrix cores, operands straight from the pages
+        if profiling:
+            if window:
+                tile_pairs = sum(sum(min(c + i + 1, window) for i in range(n)) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+                tile_keys = sum(n + min(c, window) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+            ops._note(f"portions {work.num_tiles} tiles {head_dim}/{value_dim}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+        if ops.attention_tiles(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.tile_first,
+                               work.tile_count, work.num_tiles, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
+                               head_dim=head_dim, value_dim=value_dim, page_size=page_size, scale=scale, window=window,
+                               chunk=chunk, sinks=sinks):
+            if profiling and work.num_single:
+                ops._note(f"{work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
+            ops.paged_attention_generic(
+                q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
+                num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
+                scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
             return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,

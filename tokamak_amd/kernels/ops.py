@@ -267,6 +267,10 @@ _SIGS = {
                               c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                               c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     },
+    "attention_tiles": {
+        "tk_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
+    },
     "attention_fused": {
         "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                       c_float, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -1438,6 +1442,40 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 
 
 NOT_INSTANTIATED = -2
+
+
+def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    positions: torch.Tensor, req_of_token: torch.Tensor, tile_first: torch.Tensor,
+                    tile_count: torch.Tensor, num_tiles: int, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
+                    head_dim: int, value_dim: int, page_size: int, scale: float, window: int | None = None,
+                    chunk: int | None = None, sinks: torch.Tensor | None = None) -> bool:
+    """bf16 attention of the tiles of prompt portions (up to 16 consecutive tokens of one request each) on
+    the matrix cores, for keys and values of unlike sizes (up to 512; keys in pieces of 8, values in blocks
+    of 16), any group, a window or chunks, sinks; pages of a multiple of 16 tokens.  Returns False
+    (nothing launched) for a shape it does not take."""
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, tile_first, tile_count, out, sinks)
+    n = positions.numel()
+    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype == torch.bfloat16 and page_size % 16 == 0
+            and head_dim % 8 == 0 and value_dim % 16 == 0 and max(head_dim, value_dim) <= 512):
+        return False
+    _need(not (window and chunk), "a window or chunks, not both")
+    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * value_dim, "q/out too small")
+    _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    _need(k_cache.numel() % (num_kv_heads * head_dim * page_size) == 0
+          and v_cache.numel() * head_dim == k_cache.numel() * value_dim, "cache size is not whole pages")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
+          and block_tables.dim() == 2 and tile_first.dtype == torch.int32 and tile_count.dtype == torch.int32
+          and tile_first.numel() >= num_tiles and tile_count.numel() >= num_tiles, "descriptor arrays are int32")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads), "sinks are float32 [num_heads]")
+    span = int(window or 0) if not chunk else -int(chunk)
+    status = _fn("attention_tiles", "tk_attention_tiles")(
+        _p(q), _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(positions), _p(req_of_token),
+        _p(tile_first), _p(tile_count), num_tiles, _p(out), num_heads, num_kv_heads, head_dim, value_dim, page_size,
+        float(scale), span, _p(sinks), _stream())
+    if status == NOT_INSTANTIATED:
+        return False
+    _check(status, "attention_tiles")
+    return True
 
 
 def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
