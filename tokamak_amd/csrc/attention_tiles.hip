@@ -3,9 +3,10 @@
 // pieces of 8, values in blocks of 16), any number of query heads a kv head, a window or chunks, a sink.
 // bf16 in, float32 softmax and accumulation.
 //
-// A wave owns one tile (up to 16 consecutive tokens of one request) at one query head; the four
-// waves of a block take four heads of the same tile, so what one asks of memory the others find in
-// the CU's cache.  Keys are walked 16 at a time, operands straight from the pages (no LDS):
+// A wave owns one tile (up to 16 consecutive tokens of one request) at one query head.  With fewer than
+// four query heads a kv head, the four waves of a block take four heads of the same tile and every wave
+// fetches its operands itself; with four and more, the waves of a block are heads of one kv head and
+// share the operands through LDS (second kernel below).  Keys are walked 16 at a time, operands straight from the pages (no LDS):
 //   S^T[key][token] = K[key][:] . Q[token][:]      v_mfma_f32_16x16x32_bf16, K rows as A (a lane
 //       (key, kb) reads the 16-byte piece of dims 32 c + 8 kb of its key), Q rows as B, kept in registers
 //   P^T = exp2(S^T * c - m[token])                  float32, a token's column per lane
@@ -158,6 +159,209 @@ __global__ __launch_bounds__(kHeadsPerBlock * 64) void attention_tiles_kernel(
   }
 }
 
+// The same products for kv heads with four query heads and more: a block of HB waves takes HB heads of
+// ONE kv head at one tile and shares every 16 keys' operands through LDS (each wave of the kernel above
+// fetches them from L2 for itself: with 32 heads on one kv head that is L2's rate, not the matrix
+// cores').  A stage is the 16 keys' slice of the K page (hd/8 runs of 256 bytes) and of the V page
+// (vd/16 runs of 512 bytes), copied as they lie, so the operand reads are those of the pages: a lane's
+// 16-byte key piece at ((4 c + kb) 16 + key) 8, its 8-byte value piece at ((4 d + kb) 16 + dim) 4.  Two
+// stages: the next one is fetched into registers before this one's products and written after them,
+// one barrier a stage.  Operands are read from LDS per instruction, which leaves a wave under 256
+// registers: two waves a SIMD.
+template <int KCH, int DBL, int HB>
+__global__ __launch_bounds__(HB * 64) void attention_tiles_shared_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ positions,
+    const int* __restrict__ req_of_token, const int* __restrict__ tile_first, const int* __restrict__ tile_count,
+    bf16_t* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span,
+    const float* __restrict__ sinks) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t stage_s[];   // two stages of (hd + vd) * 16 elements
+  constexpr int THREADS = HB * 64;
+  constexpr int KPT = (KCH * 64 + THREADS - 1) / THREADS;    // 16-byte pieces of K (hd / 8 * 16 = 2 hd) a thread copies
+  constexpr int VPT = (DBL * 32 + THREADS - 1) / THREADS;    // and of V (vd / 16 * 32 = 2 vd)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
+  const int group = nh / nkv, blocks_per_kv = (group + HB - 1) / HB;
+  const int kvh = blockIdx.y / blocks_per_kv;
+  const int in_group = (blockIdx.y % blocks_per_kv) * HB + wave;
+  const bool computes = in_group < group;                   // (a wave without a head still copies and waits)
+  const int head = kvh * group + (computes ? in_group : 0);
+  const int tile = blockIdx.x;
+  const int n0 = tile_first[tile], cnt = tile_count[tile];
+  const int pos0 = positions[n0];
+  const int my = min(col, cnt - 1);
+  const int pos = pos0 + my;
+  const int first = span > 0 ? max(pos - span + 1, 0) : span < 0 ? pos - pos % (-span) : 0;
+  const int lo = span > 0 ? max(pos0 - span + 1, 0) : span < 0 ? pos0 - pos0 % (-span) : 0;
+  const int hi = pos0 + cnt - 1;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t k_page = (size_t)nkv * hd * ps, v_page = (size_t)nkv * vd * ps;
+  const size_t k_head = (size_t)kvh * hd * ps, v_head = (size_t)kvh * vd * ps;
+  const int kch = (hd + 31) >> 5, dbl = vd >> 4;
+  const int k_pieces = 2 * hd, v_pieces = 2 * vd;           // 16-byte pieces of a stage
+  const int stage_elems = (hd + vd) * 16;
+
+  bf16x8 qreg[KCH];
+  const bf16_t* qp = q + ((size_t)(n0 + my) * nh + head) * hd + kb * 8;
+#pragma unroll
+  for (int c = 0; c < KCH; ++c) {
+    Frag8 f;
+    f.u = (c * 32 + kb * 8 < hd) ? *reinterpret_cast<const uint4*>(qp + c * 32) : make_uint4(0, 0, 0, 0);
+    qreg[c] = f.v;
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  float4v acc[DBL];
+#pragma unroll
+  for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  uint4 kt[KPT], vt[VPT];
+  // piece p of K: run j = p / 16 (8 dims), key p % 16; piece p of V: block d = p / 32, 16 bytes r = p % 32 of its 512
+#define TK_SFETCH(C0_)                                                                                         \
+  {                                                                                                            \
+    const int page_ = table[(C0_) / ps], off_ = (C0_) % ps;                                                    \
+    const bf16_t* kp_ = k_cache + (size_t)page_ * k_page + k_head + (size_t)off_ * 8;                          \
+    const bf16_t* vp_ = v_cache + (size_t)page_ * v_page + v_head + (size_t)(off_ >> 2) * 64;                  \
+    _Pragma("unroll") for (int i = 0; i < KPT; ++i) {                                                          \
+      const int p_ = i * THREADS + threadIdx.x;                                                                \
+      if (p_ < k_pieces) kt[i] = *reinterpret_cast<const uint4*>(kp_ + ((size_t)(p_ >> 4) * ps + (p_ & 15)) * 8); \
+    }                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < VPT; ++i) {                                                          \
+      const int p_ = i * THREADS + threadIdx.x;                                                                \
+      if (p_ < v_pieces) vt[i] = *reinterpret_cast<const uint4*>(vp_ + (size_t)(p_ >> 5) * (ps >> 2) * 64 + (p_ & 31) * 8); \
+    }                                                                                                          \
+  }
+#define TK_SSTORE(BUF_)                                                                                        \
+  {                                                                                                            \
+    bf16_t* ks_ = stage_s + (size_t)(BUF_) * stage_elems;                                                      \
+    bf16_t* vs_ = ks_ + hd * 16;                                                                               \
+    _Pragma("unroll") for (int i = 0; i < KPT; ++i) {                                                          \
+      const int p_ = i * THREADS + threadIdx.x;                                                                \
+      if (p_ < k_pieces) *reinterpret_cast<uint4*>(ks_ + (size_t)p_ * 8) = kt[i];                              \
+    }                                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < VPT; ++i) {                                                          \
+      const int p_ = i * THREADS + threadIdx.x;                                                                \
+      if (p_ < v_pieces) *reinterpret_cast<uint4*>(vs_ + (size_t)p_ * 8) = vt[i];                              \
+    }                                                                                                          \
+  }
+  const int c_first = lo & ~15;
+  TK_SFETCH(c_first)
+  TK_SSTORE(0)
+  __syncthreads();
+  int buf = 0;
+  for (int c0 = c_first; c0 <= hi; c0 += 16, buf ^= 1) {
+    const bool more = c0 + 16 <= hi;
+    if (more) TK_SFETCH(c0 + 16)
+    if (computes) {
+      const bf16_t* ks = stage_s + (size_t)buf * stage_elems;
+      const bf16_t* vs = ks + hd * 16;
+      float4v sc = {0.f, 0.f, 0.f, 0.f}, sc2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KCH; c += 2) {
+        if (c < kch) {     // (the same for every lane; a piece behind the key's end is absent from the stage: zeros)
+          Frag8 kf;
+          kf.u = (c * 32 + kb * 8 < hd) ? *reinterpret_cast<const uint4*>(ks + ((size_t)(c * 4 + kb) * 16 + col) * 8)
+                                        : make_uint4(0, 0, 0, 0);
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[c], sc, 0, 0, 0);
+        }
+        if (c + 1 < kch) {
+          Frag8 kf;
+          kf.u = ((c + 1) * 32 + kb * 8 < hd) ? *reinterpret_cast<const uint4*>(ks + ((size_t)((c + 1) * 4 + kb) * 16 + col) * 8)
+                                              : make_uint4(0, 0, 0, 0);
+          sc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[c + 1], sc2, 0, 0, 0);
+        }
+      }
+      sc += sc2;
+      float sv[4];
+      bool seen[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = c0 + kb * 4 + e;
+        seen[e] = key >= first && key <= pos;
+        sv[e] = seen[e] ? sc[e] * scale_log2 : -INFINITY;
+      }
+      float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m_run, tmax);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run - m_safe);
+      m_run = m_new;
+      float pr[4], psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pr[e] = seen[e] ? fast_exp2(sv[e] - m_safe) : 0.f;
+        psum += pr[e];
+      }
+      l_run = l_run * alpha + psum;
+      Frag4 pb;
+      pb.u = make_uint2(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]));
+      const bool edge = c0 + 15 > hi;
+      const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+#pragma unroll
+      for (int d = 0; d < DBL; ++d) {
+        if (d >= dbl) continue;
+        Frag4 vf;
+        vf.u = *reinterpret_cast<const uint2*>(vs + ((size_t)(d * 4 + kb) * 16 + col) * 4);
+        short4v tv = vf.v;
+        if (edge) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (c0 + kb * 4 + e > hi) tv[e] = 0;
+        }
+        float4v a = acc[d];
+        if (rescale) a *= alpha;
+        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(tv, pb.v, a, 0, 0, 0);
+      }
+    }
+    if (more) TK_SSTORE(buf ^ 1)
+    __syncthreads();
+  }
+#undef TK_SFETCH
+#undef TK_SSTORE
+
+  if (!computes) return;
+  float l = l_run;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (sinks) l += fast_exp2(sinks[head] * 1.4426950408889634f - m_run);
+  if (col >= cnt) return;
+  const float inv = 1.f / l;
+  bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * vd + kb * 4;
+#pragma unroll
+  for (int d = 0; d < DBL; ++d) {
+    if (d >= dbl) continue;
+    uint2 o;
+    o.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
+    o.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
+    *reinterpret_cast<uint2*>(op + d * 16) = o;
+  }
+}
+
+template <int KCH, int DBL, int HB>
+static int launch_shared(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int max_pages,
+                         const int* positions, const int* req_of_token, const int* tile_first, const int* tile_count,
+                         int num_tiles, void* out, int nh, int nkv, int hd, int vd, int ps, float scale, int span,
+                         const float* sinks, hipStream_t stream) {
+  const int group = nh / nkv;
+  const size_t lds = (size_t)2 * (hd + vd) * 16 * sizeof(bf16_t);
+  if (lds > 48 * 1024) {
+    static bool raised = false;   // per template instance
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_tiles_shared_kernel<KCH, DBL, HB>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return -2;
+      }
+      raised = true;
+    }
+  }
+  const dim3 grid(num_tiles, nkv * ((group + HB - 1) / HB));
+  if (grid.y > 65535) return -1;
+  attention_tiles_shared_kernel<KCH, DBL, HB><<<grid, HB * 64, lds, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions, req_of_token,
+      tile_first, tile_count, (bf16_t*)out, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span, sinks);
+  return launch_status();
+}
+
 }  // namespace
 
 // Tiles of up to 16 consecutive tokens of one request (tile_first, tile_count), bfloat16.  Returns -2
@@ -171,6 +375,17 @@ TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_
   if (hd > 512 || vd > 512 || (uintptr_t)q % 16 != 0 || (uintptr_t)k_cache % 16 != 0 || (uintptr_t)v_cache % 16 != 0 ||
       (uintptr_t)out % 8 != 0)
     return -2;
+  const int group = nh / nkv;
+  if (group >= 4) {
+    // the heads of a kv head share its keys and values through LDS
+#define TK_SHARED(KCH_, DBL_, HB_)                                                                              \
+  launch_shared<KCH_, DBL_, HB_>(q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, tile_first, \
+                                 tile_count, num_tiles, out, nh, nkv, hd, vd, ps, scale, span, sinks, stream)
+    if (hd <= 128 && vd <= 128) return group > 4 ? TK_SHARED(4, 8, 8) : TK_SHARED(4, 8, 4);
+    if (hd <= 256 && vd <= 256) return group > 4 ? TK_SHARED(8, 16, 8) : TK_SHARED(8, 16, 4);
+    return group > 4 ? TK_SHARED(16, 32, 8) : TK_SHARED(16, 32, 4);
+#undef TK_SHARED
+  }
   const dim3 grid(num_tiles, (nh + kHeadsPerBlock - 1) / kHeadsPerBlock);
   if (grid.y > 65535) return -1;
 #define TK_TILES(KCH_, DBL_)                                                                                   \
