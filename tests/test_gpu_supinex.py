@@ -148,6 +148,7 @@ ATTENTIONS = {
     "mid": dict(heads=4, kv_heads=1, dim=64, vdim=64, rot=64),
     "pad": dict(heads=3, kv_heads=1, dim=20, vdim=36, rot=10, window=50),
     "tiny": dict(heads=2, kv_heads=2, dim=6, vdim=2, rot=6),
+    "g9": dict(heads=18, kv_heads=2, dim=24, vdim=32, rot=8),
 }
 
 
@@ -172,10 +173,11 @@ def attention_part(m, width, dtype, value_mix=None):
 def test_sink_attention_alone_with_mixed_values(dtype, name):
     """Two layers over the same tokens, the second mixing the first one's values into its own: a
     portion from position zero, one that ends inside a page, two tokens, then single tokens; pages
-    scattered.  Heads of 64 and 128 with pages of 16 run on the matrix cores in bfloat16."""
+    scattered.  Heads of 64 and 128 with pages of 16 run on the tuned matrix-core kernels in bfloat16, other
+    sizes with pages of 16 on the ones that take any size (nine heads a kv head: single tokens too)."""
     a = ATTENTIONS[name]
     width = 64
-    page = 16 if a["dim"] >= 64 else 8
+    page = 16 if a["dim"] >= 64 or name in ("g9", "pad") else 8
     cfg = model_json([attention(**a, v_mix=True), attention(**a, v_mix=True)], width=width)
     m = cfg["layers"][0]["mixer"]
     w = random_weights(cfg, seed=a["dim"])
@@ -268,6 +270,7 @@ LATENTS = {
     "no-window": dict(heads=5, dim=32, rot_dim=16, vdim=24, kv_rank=80, window=None, base=1e5),
     "no-rot": dict(heads=2, dim=16, rot_dim=8, vdim=8, kv_rank=12, window=64, rot=0),
     "big": dict(heads=4, dim=64, rot_dim=32, vdim=64, kv_rank=160, window=100),
+    "many-heads": dict(heads=20, dim=16, rot_dim=8, vdim=16, kv_rank=40, window=70),
 }
 
 
@@ -279,7 +282,7 @@ def test_latent_attention_alone(dtype, name):
     from tokamak_amd.config import get_part
 
     a = LATENTS[name]
-    width, eps, page = 64, 1e-5, 8
+    width, eps, page = 64, 1e-5, 16 if name in ("big", "many-heads", "odd") else 8
     cfg = model_json([latent(**a)], width=width, eps=eps)
     m = cfg["layers"][0]["mixer"]
     w = random_weights(cfg, seed=a["kv_rank"])
@@ -384,7 +387,7 @@ def test_routed_experts_with_softmax_scores_on_the_outputs(dtype, width, ff, n, 
 
 # -- whole models -------------------------------------------------------------------
 SHAPES = {
-    "base": dict(cfg=model_json([attention(v_mix=True, mlp=dense(40)), latent(), attention(v_mix=True), latent(window=45, mlp=dense(24)),
+    "base": dict(cfg=model_json([attention(v_mix=True, mlp=dense(40)), latent(), attention(v_mix=True), latent(heads=9, window=45, mlp=dense(24)),
                                  attention(v_mix=True, rot=16)]), page=16),
     "odd": dict(cfg=model_json([latent(heads=3, dim=20, rot_dim=12, vdim=36, kv_rank=45, window=7, rot=6, yarn=(4.0, 32.0, 8.0, 1.0),
                                        mlp=experts(5, 1, 24)),

@@ -1,7 +1,8 @@
 // Paged attention of prompt portions on the matrix cores for the shapes the tuned kernels of
 // attention_mfma.hip do not take: keys and values of unlike sizes (up to 512 channels each, keys in
 // pieces of 8, values in blocks of 16), any number of query heads a kv head, a window or chunks, a sink.
-// bf16 in, float32 softmax and accumulation.
+// bf16 in, float32 softmax and accumulation.  Tokens that run alone have a form of their own (third
+// kernel below) where a kv head has many query heads.
 //
 // A wave owns one tile (up to 16 consecutive tokens of one request) at one query head.  With fewer than
 // four query heads a kv head, the four waves of a block take four heads of the same tile and every wave
@@ -362,6 +363,163 @@ static int launch_shared(const void* q, const void* k_cache, const void* v_cache
   return launch_status();
 }
 
+// Tokens that run alone (decode) at kv heads with many query heads: the 16 columns of a wave's products
+// are 16 HEADS of one kv head at one token, so a key or value fetched once serves them all.  The token's
+// visible keys are walked 16 at a time; step t goes to wave t % (4 nsplit) of the token's nsplit blocks
+// of four waves, operands straight from the pages.  Every wave leaves an unnormalised partial result
+// (its maximum, its sum, its output) and a second kernel merges a head's partials in their order and
+// adds the sink: no wave waits for another.
+template <int KCH, int DBL>
+__global__ __launch_bounds__(256) void attention_heads_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ positions,
+    const int* __restrict__ req_of_token, const int* __restrict__ single, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int nsplit, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
+  const int group = nh / nkv, pieces = (group + 15) >> 4;
+  const int kvh = blockIdx.y / pieces, in_group = (blockIdx.y % pieces) * 16 + col;
+  const bool c_valid = in_group < group;
+  const int head = kvh * group + min(in_group, group - 1);
+  const int item = blockIdx.x, n0 = single[item];
+  const int pos = positions[n0];
+  const int first = span > 0 ? max(pos - span + 1, 0) : span < 0 ? pos - pos % (-span) : 0;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t k_page = (size_t)nkv * hd * ps, v_page = (size_t)nkv * vd * ps;
+  const size_t k_head = (size_t)kvh * hd * ps, v_head = (size_t)kvh * vd * ps;
+  const int kch = (hd + 31) >> 5, dbl = vd >> 4;
+  const int parts = nsplit * 4, part = blockIdx.z * 4 + wave;
+
+  bf16x8 qreg[KCH];
+  const bf16_t* qp = q + ((size_t)n0 * nh + head) * hd + kb * 8;
+#pragma unroll
+  for (int c = 0; c < KCH; ++c) {
+    Frag8 f;
+    f.u = (c * 32 + kb * 8 < hd) ? *reinterpret_cast<const uint4*>(qp + c * 32) : make_uint4(0, 0, 0, 0);
+    qreg[c] = f.v;
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  float4v acc[DBL];
+#pragma unroll
+  for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  for (int c0 = (first & ~15) + part * 16; c0 <= pos; c0 += parts * 16) {
+    const int page = table[c0 / ps], off = c0 % ps;
+    const bf16_t* kp = k_cache + (size_t)page * k_page + k_head + (size_t)(off + col) * 8;
+    const bf16_t* vp = v_cache + (size_t)page * v_page + v_head + (size_t)((off >> 2) + kb) * 64 + col * 4;
+    Frag8 kreg[KCH];
+#pragma unroll
+    for (int c = 0; c < KCH; ++c)
+      kreg[c].u = (c * 32 + kb * 8 < hd) ? *reinterpret_cast<const uint4*>(kp + (size_t)(c * 4 + kb) * ps * 8)
+                                         : make_uint4(0, 0, 0, 0);
+    Frag4 vreg[DBL];
+#pragma unroll
+    for (int d = 0; d < DBL; ++d)
+      vreg[d].u = d < dbl ? *reinterpret_cast<const uint2*>(vp + (size_t)d * (ps >> 2) * 64) : make_uint2(0, 0);
+    float4v sc = {0.f, 0.f, 0.f, 0.f}, sc2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KCH; c += 2) {
+      if (c < kch) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[c].v, qreg[c], sc, 0, 0, 0);
+      if (c + 1 < kch) sc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[c + 1].v, qreg[c + 1], sc2, 0, 0, 0);
+    }
+    sc += sc2;
+    float sv[4];
+    bool seen[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int key = c0 + kb * 4 + e;
+      seen[e] = key >= first && key <= pos;
+      sv[e] = seen[e] ? sc[e] * scale_log2 : -INFINITY;
+    }
+    float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m_run, tmax);   // finite: a step holds at least one visible key
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
+    float pr[4], psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      pr[e] = seen[e] ? fast_exp2(sv[e] - m_new) : 0.f;
+      psum += pr[e];
+    }
+    l_run = l_run * alpha + psum;
+    Frag4 pb;
+    pb.u = make_uint2(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]));
+    const bool edge = c0 + 15 > pos;
+#pragma unroll
+    for (int d = 0; d < DBL; ++d) {
+      if (d >= dbl) continue;
+      short4v tv = vreg[d].v;
+      if (edge) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (c0 + kb * 4 + e > pos) tv[e] = 0;
+      }
+      float4v a = acc[d];
+      a *= alpha;
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(tv, pb.v, a, 0, 0, 0);
+    }
+  }
+  float l = l_run;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (!c_valid) return;
+  // partial rows [item][head][part]: (maximum, sum), then the output
+  const size_t prow = ((size_t)item * nh + head) * parts + part;
+  if (kb == 0) {
+    part_ml[prow * 2] = m_run;
+    part_ml[prow * 2 + 1] = l;
+  }
+  float* po = part_o + prow * vd + kb * 4;
+#pragma unroll
+  for (int d = 0; d < DBL; ++d) {
+    if (d >= dbl) continue;
+    *reinterpret_cast<float4*>(po + d * 16) = make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
+  }
+}
+
+// out[token][head] = sum_p w_p o_p / (sum_p w_p l_p + exp(sink)), w_p = exp2(m_p - max m); a part without
+// keys has m = -inf and weighs nothing (its output is not read).  A block a (token, head): lane p of the
+// first wave takes part p's maximum and sum (up to 64 parts), then a thread a value channel, the parts'
+// outputs asked for eight at a time and added in their order.
+__global__ __launch_bounds__(256) void attention_heads_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ single,
+    bf16_t* __restrict__ out, int parts, int nh, int vd, const float* __restrict__ sinks) {
+  __shared__ float w_s[64];
+  __shared__ float inv_s;
+  const int item = blockIdx.x, head = blockIdx.y;
+  const size_t row = ((size_t)item * nh + head) * parts;
+  if (threadIdx.x < 64) {
+    const int p = threadIdx.x;
+    const float m = p < parts ? part_ml[(row + p) * 2] : -INFINITY;
+    const float l = p < parts ? part_ml[(row + p) * 2 + 1] : 0.f;
+    const float mx = wave_max(m);                       // finite: the part that holds the token's own key
+    const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx);
+    float denom = wave_sum(w * (m == -INFINITY ? 0.f : l));
+    if (sinks) denom += fast_exp2(sinks[head] * 1.4426950408889634f - mx);
+    w_s[p] = w;
+    if (p == 0) inv_s = 1.f / denom;
+  }
+  __syncthreads();
+  const float inv = inv_s;
+  bf16_t* op = out + ((size_t)single[item] * nh + head) * vd;
+  const float* po = part_o + row * vd;
+  for (int d = threadIdx.x; d < vd; d += blockDim.x) {
+    float o = 0.f;
+    for (int p0 = 0; p0 < parts; p0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = p0 + u;
+        v[u] = (p < parts && w_s[p] != 0.f) ? po[(size_t)p * vd + d] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) o = fmaf(p0 + u < parts ? w_s[p0 + u] : 0.f, v[u], o);
+    }
+    op[d] = float_to_bf16(o * inv);
+  }
+}
+
 }  // namespace
 
 // Tiles of up to 16 consecutive tokens of one request (tile_first, tile_count), bfloat16.  Returns -2
@@ -400,4 +558,32 @@ TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_
   return launch_status();
 }
 
+// Single tokens (`single`: their rows, num_single of them), bfloat16, for kv heads with many query heads.
+// part_o: float32 [num_single * nh * 4 nsplit * vd], part_ml: float32 [num_single * nh * 4 nsplit * 2].
+TK_API int tk_attention_heads(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
+                              int max_pages, const int* positions, const int* req_of_token, const int* single,
+                              int num_single, void* out, float* part_o, float* part_ml, int nsplit, int nh, int nkv,
+                              int hd, int vd, int ps, float scale, int span, const float* sinks, hipStream_t stream) {
+  if (num_single <= 0) return 0;
+  if (nkv <= 0 || nh % nkv != 0 || hd < 8 || hd % 8 != 0 || vd < 16 || vd % 16 != 0 || ps < 16 || ps % 16 != 0) return -2;
+  if (hd > 512 || vd > 512 || (uintptr_t)q % 16 != 0 || (uintptr_t)k_cache % 16 != 0 || (uintptr_t)v_cache % 16 != 0 ||
+      (uintptr_t)part_o % 16 != 0 || nsplit < 1 || nsplit > 16 || nh > 65535)    // (the merge: up to 64 parts)
+    return -2;
+  const int group = nh / nkv;
+  const dim3 grid(num_single, nkv * ((group + 15) / 16), nsplit);
+  if (grid.y > 65535) return -1;
+#define TK_HEADS(KCH_, DBL_)                                                                                  \
+  attention_heads_kernel<KCH_, DBL_><<<grid, 256, 0, stream>>>(                                               \
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,   \
+      req_of_token, single, part_o, part_ml, nsplit, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span)
+  if (hd <= 128 && vd <= 128) TK_HEADS(4, 8);
+  else if (hd <= 256 && vd <= 256) TK_HEADS(8, 16);
+  else TK_HEADS(16, 32);
+#undef TK_HEADS
+  attention_heads_merge_kernel<<<dim3(num_single, nh), vd <= 64 ? 64 : vd <= 128 ? 128 : 256, 0, stream>>>(  // (whole waves)
+      part_o, part_ml, single, (bf16_t*)out, nsplit * 4, nh, vd, sinks);
+  return launch_status();
+}
+
 TK_SLOTS(tk_attention_tiles)
+TK_SLOTS(tk_attention_heads)

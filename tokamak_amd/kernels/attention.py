@@ -27,6 +27,8 @@ WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles 
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
 GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays
 GROUP_FILL = 128                # ... if its blocks times their shares of the keys are at least this many (half the CUs)
+HEADS_FORM_FROM_GROUP = 8       # query heads a kv head from which tokens that run alone take ops.attention_heads (the
+                                # heads are a product's 16 columns: with fewer, most of a product is idle)
 TILES_ON_MATRIX_CORES = True    # bfloat16 portions that the tuned kernels do not take: csrc/attention_tiles.hip rather than
                                 # the generic kernel (tests of the generic kernel's own tiles switch this off)
 
@@ -141,6 +143,15 @@ def check_page_size(page_size: int) -> None:
     the key layout in pieces of 8 numbers, and the generic kernel walks pages 8 keys at a time."""
     if page_size < 8 or page_size % 8:
         raise ValueError(f"page_size must be a multiple of 8 for the attention kernels, got {page_size}")
+
+
+def heads_form_splits(num_single: int, num_kv_heads: int, group: int, max_len: int, window, chunk) -> int:
+    """Blocks of four waves that share a token's visible keys in ``ops.attention_heads``: enough to give
+    every CU a block, but no wave fewer than two steps of 16 keys."""
+    keys = min(max_len, window or max_len, chunk or max_len)
+    steps = -(-keys // 16) + 1
+    blocks = max(1, num_single * num_kv_heads * -(-group // 16))
+    return max(1, min(-(-steps // 8), 256 // blocks, 16))     # (the merge takes up to 64 partial results)
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -329,25 +340,38 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
                 num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
                 scale=scale, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
             return
-    if TILES_ON_MATRIX_CORES and work.num_tiles and q.dtype == torch.bfloat16 and page_size % 16 == 0:
-        # bfloat16 portions at shapes the tuned kernels do not take (unlike key and value sizes, other head
-        # sizes, a window): tiles of 16 tokens on the matrix cores, operands straight from the pages
-        if profiling:
-            if window:
-                tile_pairs = sum(sum(min(c + i + 1, window) for i in range(n)) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
-                tile_keys = sum(n + min(c, window) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
-            ops._note(f"portions {work.num_tiles} tiles {head_dim}/{value_dim}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
-        if ops.attention_tiles(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.tile_first,
-                               work.tile_count, work.num_tiles, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
-                               head_dim=head_dim, value_dim=value_dim, page_size=page_size, scale=scale, window=window,
-                               chunk=chunk, sinks=sinks):
-            if profiling and work.num_single:
-                ops._note(f"{work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
+    group = num_heads // num_kv_heads
+    heads_form = group >= HEADS_FORM_FROM_GROUP and work.num_single > 0
+    if (TILES_ON_MATRIX_CORES and (work.num_tiles or heads_form)
+            and ops.attention_tiles_fit(q.dtype, head_dim, value_dim, page_size)):
+        # bfloat16 at shapes the tuned kernels do not take (unlike key and value sizes, other head sizes, a
+        # window): on the matrix cores with operands straight from the pages; portions in tiles of 16 tokens,
+        # tokens that run alone with the heads of a kv head as a product's columns where there are enough
+        if profiling and window:
+            tile_pairs = sum(sum(min(c + i + 1, window) for i in range(n)) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+            tile_keys = sum(n + min(c, window) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+            decode_keys = sum(min(c + 1, window) for c, n in zip(batch.ctx_lens, batch.q_lens) if n == 1)
+        if work.num_tiles:
+            if profiling:
+                ops._note(f"portions {work.num_tiles} tiles {head_dim}/{value_dim}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+            if not ops.attention_tiles(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.tile_first,
+                                       work.tile_count, work.num_tiles, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
+                                       head_dim=head_dim, value_dim=value_dim, page_size=page_size, scale=scale, window=window,
+                                       chunk=chunk, sinks=sinks):
+                raise ops.KernelError("the tile kernel refused a shape it was asked about")
+        if profiling and work.num_single:
+            ops._note(f"{work.num_single} tokens {head_dim}/{value_dim}", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
+        if heads_form:
+            ops.attention_heads(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.single,
+                                work.num_single, out, num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
+                                value_dim=value_dim, page_size=page_size, scale=scale, window=window, chunk=chunk, sinks=sinks,
+                                num_splits=heads_form_splits(work.num_single, num_kv_heads, group, work.max_single_len, window, chunk))
+        elif work.num_single:
             ops.paged_attention_generic(
                 q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
                 num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
                 scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
-            return
+        return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
                   (decode_keys + tile_pairs) * flops_per_pair)

@@ -270,6 +270,9 @@ _SIGS = {
     "attention_tiles": {
         "tk_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
+        "tk_attention_heads": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                               c_void_p, c_void_p],
     },
     "attention_fused": {
         "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -1534,6 +1537,44 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
         return False
     _check(status, "attention_mfma")
     return True
+
+
+def attention_tiles_fit(dtype: torch.dtype, head_dim: int, value_dim: int, page_size: int) -> bool:
+    """Whether ``attention_tiles`` and ``attention_heads`` take the shape."""
+    return (dtype == torch.bfloat16 and page_size % 16 == 0 and head_dim % 8 == 0 and value_dim % 16 == 0
+            and 8 <= head_dim <= 512 and 16 <= value_dim <= 512)
+
+
+def attention_heads(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    positions: torch.Tensor, req_of_token: torch.Tensor, single: torch.Tensor, num_single: int,
+                    out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                    page_size: int, scale: float, num_splits: int, window: int | None = None,
+                    chunk: int | None = None, sinks: torch.Tensor | None = None) -> None:
+    """bf16 attention of tokens that run alone (``single``: their rows) on the matrix cores, the 16 columns of
+    a product being 16 query heads of one kv head, for the shapes of ``attention_tiles``.  Each token's visible
+    keys are dealt, 16 at a time, to the four waves of ``num_splits`` blocks; a second kernel merges the waves'
+    partial results and adds the sinks."""
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, single, out, sinks)
+    n = positions.numel()
+    _need(attention_tiles_fit(q.dtype, head_dim, value_dim, page_size) and k_cache.dtype == v_cache.dtype == out.dtype == q.dtype,
+          "attention_heads takes bfloat16, pages of a multiple of 16, keys in pieces of 8, values in blocks of 16")
+    _need(not (window and chunk), "a window or chunks, not both")
+    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * value_dim, "q/out too small")
+    _need(num_heads % num_kv_heads == 0 and 1 <= num_splits <= 16, "bad head counts, or more than 16 splits")
+    _need(k_cache.numel() % (num_kv_heads * head_dim * page_size) == 0
+          and v_cache.numel() * head_dim == k_cache.numel() * value_dim, "cache size is not whole pages")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
+          and block_tables.dim() == 2 and single.dtype == torch.int32 and single.numel() >= num_single > 0,
+          "descriptor arrays are int32")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads), "sinks are float32 [num_heads]")
+    rows = num_single * num_heads * num_splits * 4
+    part_o = torch.empty((rows, value_dim), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((rows, 2), dtype=torch.float32, device=q.device)
+    span = int(window or 0) if not chunk else -int(chunk)
+    _check(_fn("attention_tiles", "tk_attention_heads")(
+        _p(q), _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(positions), _p(req_of_token),
+        _p(single), num_single, _p(out), _p(part_o), _p(part_ml), num_splits, num_heads, num_kv_heads, head_dim,
+        value_dim, page_size, float(scale), span, _p(sinks), _stream()), "attention_heads")
 
 
 FUSED_DECODE_MAX_GROUP = 14   # query heads per kv head the fused decode kernel takes (two waves make the key and value)
