@@ -246,7 +246,13 @@ struct RowScale {
   const float* sumsq;  // [slabs][M]: sums of squares of the rows over slabs of columns; nullptr: no scaling
   int slabs;
   float eps;
+  int act;             // the gated form's activation: 0 silu, 1 the tanh form of gelu
 };
+
+__device__ __forceinline__ float gate_act(float z, int act) {
+  if (act == 0) return z / (1.f + __expf(-z));
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
 
 template <int MT, typename TO, bool GATED, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
@@ -434,10 +440,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       const float4 u = *reinterpret_cast<const float4*>(up + ((size_t)(wave * MT + j) * 64 + lane) * 4);
-      acc[j][0] = acc[j][0] / (1.f + __expf(-acc[j][0])) * u.x;
-      acc[j][1] = acc[j][1] / (1.f + __expf(-acc[j][1])) * u.y;
-      acc[j][2] = acc[j][2] / (1.f + __expf(-acc[j][2])) * u.z;
-      acc[j][3] = acc[j][3] / (1.f + __expf(-acc[j][3])) * u.w;
+      acc[j][0] = gate_act(acc[j][0], scale.act) * u.x;
+      acc[j][1] = gate_act(acc[j][1], scale.act) * u.y;
+      acc[j][2] = gate_act(acc[j][2], scale.act) * u.z;
+      acc[j][3] = gate_act(acc[j][3], scale.act) * u.w;
     }
   }
 
@@ -507,7 +513,7 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
   if (M <= 0 || N <= 0) return 0;
   if (M > (waves >= 8 ? 128 : 64) || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
   if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
-  const RowScale scale{sumsq, slabs, eps};
+  const RowScale scale{sumsq, slabs, eps, 0};
   if (splits > 1 && out_dtype != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   const int cps = (total_chunks + splits - 1) / splits;
@@ -518,16 +524,18 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
   return status == 0 ? ks : (status > 0 ? -status : status);
 }
 
-// C[M, N] = silu(A W_gate^T) * (A W_up^T) with W = [W_gate; W_up] of 2N rows; bfloat16 out.
+// C[M, N] = act(A W_gate^T) * (A W_up^T) with W = [W_gate; W_up] of 2N rows; bfloat16 out.  act: 0 silu, 1 the
+// tanh form of gelu.
 TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, int N, int K, long lda,
                                  long ldw, long ldc, int waves, const float* sumsq, int slabs, float eps,
-                                 hipStream_t stream) {
+                                 int act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (act != 0 && act != 1) return -1;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
   if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,
-                                     RowScale{sumsq, slabs, eps}, stream);
+                                     RowScale{sumsq, slabs, eps, act}, stream);
 }
 
 // the same entry points in slot form (slots.h), for launch lists

@@ -135,15 +135,22 @@ def _sink_fits(sink: StreamSink, m: int, n: int) -> bool:
 def gated_linear(x: torch.Tensor | DeferredNorm, gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
     """act(x @ gate^T) * (x @ up^T) for ``gate_up`` = [gate; up] ([2I, K]) -> [M, I].
 
-    bfloat16 with up to 64 rows and the SiLU gate: one fused weight-streaming kernel.  Otherwise
-    the product, then the gate kernel (``activation``: "silu" or "gelu_tanh").
+    bfloat16 with up to 64 rows: one fused weight-streaming kernel (the whole-K form for very small
+    matrices has the SiLU gate only).  Otherwise the product, then the gate kernel (``activation``:
+    "silu" or "gelu_tanh").
     """
     m = x.shape[0]
     if activation != "silu":
         if isinstance(x, DeferredNorm):
             x = x.materialize()
         out = torch.empty((m, gate_up.shape[0] // 2), dtype=x.dtype, device=x.device)
-        if m:
+        if m == 0:
+            return out
+        from tokamak_amd.kernels import gemm_bf16
+
+        if x.dtype == torch.bfloat16 and m <= 64 and gemm_bf16.skinny_fits(x, gate_up):
+            ops.gemm_stream_swiglu(x, gate_up, out, activation=activation)
+        else:
             ops.silu_mul(linear(x, gate_up), out, activation)
         return out
     inter = gate_up.shape[0] // 2

@@ -234,7 +234,7 @@ _SIGS = {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_long, c_int, c_void_p, c_int, c_float, c_void_p],
         "tk_gemm_stream_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long,
-                                  c_int, c_void_p, c_int, c_float, c_void_p],
+                                  c_int, c_void_p, c_int, c_float, c_int, c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
     },
@@ -1174,10 +1174,12 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
 
 
 def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, waves: int = 0,
-                       sumsq: torch.Tensor | None = None, eps: float = 0.0) -> None:
-    """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for M <= 64: the gate and up
-    projections and the SiLU product in one weight-streaming kernel (bfloat16).  ``sumsq``,
-    ``eps``: the rows' scale, applied to both products before the gate, as in ``gemm_stream``."""
+                       sumsq: torch.Tensor | None = None, eps: float = 0.0, activation: str = "silu") -> None:
+    """out[M, I] = act(a @ w[:I]^T) * (a @ w[I:]^T) for M <= 64: the gate and up
+    projections and the gate product in one weight-streaming kernel (bfloat16); act is silu or the tanh
+    form of gelu.  ``sumsq``, ``eps``: the rows' scale, applied to both products before the gate, as in
+    ``gemm_stream``."""
+    _need(activation in GATE_ACTIVATIONS, f"the gate's activation is one of {sorted(GATE_ACTIVATIONS)}")
     for t in (a, w, out):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
@@ -1190,7 +1192,8 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
                                                      w.stride(0), out.stride(0), waves,
-                                                     _p(sumsq), slabs, float(eps), _stream()), "gemm_stream_swiglu")
+                                                     _p(sumsq), slabs, float(eps), GATE_ACTIVATIONS[activation],
+                                                     _stream()), "gemm_stream_swiglu")
 
 
 WHOLEK_MAX_ROWS = 16    # rows of activations that the whole-K product takes
