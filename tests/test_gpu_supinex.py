@@ -86,7 +86,7 @@ def fresh_store(part, page, pages, dtype, fill):
 
 # -- mechanisms alone -------------------------------------------------------------
 @BOTH
-@pytest.mark.parametrize("width", [64, 50, 320, 4100])
+@pytest.mark.parametrize("width", [64, 50, 328, 4100])
 def test_layer_norm_adds_both_branches_once(dtype, width):
     """x + (a + b) with a in the compute dtype and b as float32 partial sums, the stream written back;
     rows picked by index leave the stream alone; a norm without anything to add."""

@@ -80,9 +80,9 @@ def test_optional_keys_may_be_absent():
     assert made.layers[0].role("mixer").spec["num_kv_heads"] == 4
 
 
-@pytest.mark.parametrize("rot", [dict(base=10000.0, dims=16), dict(base=250000.0, dims=32, scaling=dict(factor=2.0, original=512, fast=32.0, slow=1.0)),
+@pytest.mark.parametrize("rot", [dict(base=10000.0, dims=16), dict(base=120000.0, dims=40, scaling=dict(factor=3.0, original=256, fast=16.0, slow=2.0)),
                                  dict(base=500.0, dims=8, scaling=dict(factor=8.0, original=16, fast=4.0, slow=0.5)),
-                                 dict(base=1e6, dims=64, scaling=dict(factor=40.0, original=4096, fast=32.0, slow=1.0))])
+                                 dict(base=1e6, dims=64, scaling=dict(factor=40.0, original=4096, fast=24.0, slow=2.0))])
 def test_stretched_frequencies_match_the_plain_ones(rot):
     from tokamak_amd.parts.rotary import yarn_frequencies
 

@@ -322,7 +322,7 @@ def _shape(vocab, width, pairs, *, heads, kv, dim, latent_heads, latent_dim, rot
     feed-forward is dense, the others are mixtures of experts."""
     att = AttentionConfig(heads, kv, dim, dim, float(dim) ** -0.5, RotaryConfig(5e5, dim // 2), None, True)
     lat = LatentConfig(latent_heads, latent_dim, rot_dim, latent_dim, rank, float(latent_dim + rot_dim) ** -0.5,
-                       RotaryConfig(1e4, rot_dim, YarnScaling(8.0, 4096.0, 32.0, 1.0)), window)
+                       RotaryConfig(1e4, rot_dim, YarnScaling(8.0, 4096.0, 24.0, 2.0)), window)
     moe = ExpertsConfig(experts, top, expert_ff)
     layers = [SupinexLayer(att, DenseConfig(ff)), SupinexLayer(lat, moe)] + [SupinexLayer(att, moe), SupinexLayer(lat, moe)] * (pairs - 1)
     return SupinexConfig(NAME, vocab, width, 1e-5, tuple(layers))
