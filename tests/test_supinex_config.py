@@ -172,3 +172,20 @@ def test_plain_experts_with_all_chosen_is_the_softmax_weighted_sum():
                for e in range(3))
     assert torch.allclose(got, want, atol=1e-12)
     assert oracle_logits(cfg, random_weights(cfg, 5), [1, 2, 3]).shape == (3, cfg["vocab"])
+
+
+def test_key_splits_of_single_tokens_with_many_heads():
+    """Blocks that share a token's keys in the heads-as-columns form: none for short contexts, more the
+    fewer tokens there are, a wave never under two steps of 16 keys, at most 16 (the merge's 64 parts)."""
+    from tokamak_amd.kernels.attention import heads_form_splits
+
+    assert heads_form_splits(1, 1, 8, 20, None, None) == 1
+    assert heads_form_splits(8, 1, 32, 2112, 1024, None) == 9          # 65 steps of the window, two pieces of 16 heads
+    assert heads_form_splits(8, 1, 32, 2112, None, None) == 16
+    assert heads_form_splits(1, 1, 16, 100000, None, None) == 16
+    assert heads_form_splits(64, 2, 16, 4000, None, None) == 2
+    assert heads_form_splits(300, 4, 8, 4000, None, None) == 1
+    for tokens in (1, 3, 17, 200):
+        for keys in (1, 15, 16, 17, 500, 5000):
+            n = heads_form_splits(tokens, 2, 12, keys, None, 64)
+            assert 1 <= n <= 16 and (n == 1 or n * 8 <= min(keys, 64) // 16 + 2 + 8)

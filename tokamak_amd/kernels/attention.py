@@ -303,6 +303,10 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     single tokens (which read a chunk at most) and everything else in the generic kernel.
     ``sinks``: float32 [num_heads], one more term exp(sinks[a]) of head a's denominator, added where
     a row's sums are complete (every kernel has it).
+    bfloat16 at other shapes (key and value sizes that differ or are not 64 or 128, a window), with pages
+    of a multiple of 16 tokens: the portions' tiles on the matrix cores with operands straight from the
+    pages, or through LDS for the heads of one kv head (``ops.attention_tiles``); tokens that run alone
+    too where a kv head has eight query heads and more (``ops.attention_heads``).
     """
     value_dim = head_dim if value_dim is None else value_dim
     work = work_of(batch)
