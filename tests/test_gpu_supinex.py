@@ -387,7 +387,7 @@ def test_routed_experts_with_softmax_scores_on_the_outputs(dtype, width, ff, n, 
 
 # -- whole models -------------------------------------------------------------------
 SHAPES = {
-    "base": dict(cfg=model_json([attention(v_mix=True, mlp=dense(40)), latent(), attention(v_mix=True), latent(heads=9, window=45, mlp=dense(24)),
+    "base": dict(cfg=model_json([attention(v_mix=True, mlp=dense(40)), latent(), attention(v_mix=True), latent(heads=9, window=150, mlp=dense(24)),
                                  attention(v_mix=True, rot=16)]), page=16),
     "odd": dict(cfg=model_json([latent(heads=3, dim=20, rot_dim=12, vdim=36, kv_rank=45, window=7, rot=6, yarn=(4.0, 32.0, 8.0, 1.0),
                                        mlp=experts(5, 1, 24)),

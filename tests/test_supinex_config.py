@@ -179,7 +179,10 @@ def test_key_splits_of_single_tokens_with_many_heads():
     fewer tokens there are, a wave never under two steps of 16 keys, at most 16 (the merge's 64 parts)."""
     from tokamak_amd.kernels.attention import heads_form_splits
 
-    assert heads_form_splits(1, 1, 8, 20, None, None) == 1
+    assert heads_form_splits(1, 1, 8, 20, 30, None) == 1
+    # the context counts as recorded steps round it, so a step splits alike recorded or not
+    assert heads_form_splits(1, 1, 8, 20, None, None) == heads_form_splits(1, 1, 8, 256, None, None)
+    assert heads_form_splits(2, 1, 8, 257, None, None) == heads_form_splits(2, 1, 8, 320, None, None)
     assert heads_form_splits(8, 1, 32, 2112, 1024, None) == 9          # 65 steps of the window, two pieces of 16 heads
     assert heads_form_splits(8, 1, 32, 2112, None, None) == 16
     assert heads_form_splits(1, 1, 16, 100000, None, None) == 16

@@ -148,6 +148,8 @@ def check_page_size(page_size: int) -> None:
 def heads_form_splits(num_single: int, num_kv_heads: int, group: int, max_len: int, window, chunk) -> int:
     """Blocks of four waves that share a token's visible keys in ``ops.attention_heads``: enough to give
     every CU a block, but no wave fewer than two steps of 16 keys."""
+    # (the longest context rounded as recorded steps round it: a step computes the same bits recorded or not)
+    max_len = quarter_octave_at_least(max_len, 256)
     keys = min(max_len, window or max_len, chunk or max_len)
     steps = -(-keys // 16) + 1
     blocks = max(1, num_single * num_kv_heads * -(-group // 16))
