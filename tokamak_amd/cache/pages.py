@@ -25,11 +25,14 @@ class OutOfPagesError(RuntimeError):
 class CacheGroupSpec:
     """``slots``: cache slots stored in this group's pages.  ``window``: None
     keeps every token; W keeps only what a query may still see when each query
-    sees the last W positions (itself included)."""
+    sees the last W positions (itself included).  ``keep_first``: with a window, every
+    query also sees the first so many positions of its sequence: the pages that hold
+    them are never given back while the request lives."""
 
     name: str
     slots: tuple[int, ...]
     window: int | None = None
+    keep_first: int = 0
 
 
 class PagePool:
@@ -89,7 +92,8 @@ class GroupTables:
         self.page_size = page_size
         self.pool = PagePool(num_pages)
         self.tables: dict[object, list[int]] = {}
-        self.first_live: dict[object, int] = {}  # logical pages below this were released
+        self.first_live: dict[object, int] = {}  # logical pages below this (and behind the kept first ones) were released
+        self.kept_pages = -(-max(0, spec.keep_first) // page_size)   # logical pages that hold the kept first positions
 
     def pages_needed(self, num_tokens: int) -> int:
         if num_tokens < 0:
@@ -109,7 +113,7 @@ class GroupTables:
         table = self.tables.get(request)
         if table is None:
             return 0
-        lo = self.first_live.get(request, 0)
+        lo = self.first_live.get(request, self.kept_pages)
         hi = min(max(first_needed_position // self.page_size, lo), len(table))
         self.pool.give_back(table[i] for i in range(lo, hi))
         for i in range(lo, hi):
@@ -123,8 +127,8 @@ class GroupTables:
         table = self.tables.get(request)
         if table is None:
             return 0
-        lo = self.first_live.get(request, 0)
-        return min(max(first_needed_position // self.page_size, lo), len(table)) - lo
+        lo = self.first_live.get(request, self.kept_pages)
+        return max(0, min(max(first_needed_position // self.page_size, lo), len(table)) - lo)
 
     def free(self, request) -> None:
         table = self.tables.pop(request, None)

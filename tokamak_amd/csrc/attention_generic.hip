@@ -17,7 +17,9 @@
 //
 // Keys and values may differ in size (hd and vd).  What a query sees besides causality is given
 // by `span`: 0 everything before it, W > 0 the last W positions, -C < 0 the positions of its own
-// chunk of C (chunks counted from position 0 of the sequence).
+// chunk of C (chunks counted from position 0 of the sequence).  With a window, `keep` > 0 leaves the
+// first `keep` positions of the sequence visible as well, whatever the distance (they keep their places:
+// a round of 64 keys still goes to the wave its index names).
 //
 // Cache pages: K [nkv][hd/8][ps][8], V [nkv][vd/16][ps/4][16][4] (see elementwise.hip).
 #include "common.h"
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, GenericItems items, T* __restrict__ out, int nh, int nkv,
-    int hd, int vd, int ps, int max_pages, float scale, int span, const float* __restrict__ sinks) {
+    int hd, int vd, int ps, int max_pages, float scale, int span, int keep, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) float q_s[QT][kMaxHd];
   __shared__ __attribute__((aligned(16))) float p_s[kWaves][kWave][QT];
   __shared__ long base_s[kWaves][kWave];  // where a key's values lie (a quad's, for tokens that run alone), or -1
@@ -131,10 +133,12 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
   }
 
   // this wave's rounds: those whose index is wave modulo kWaves, from the one that holds lo
-  const int round0 = lo / kWave;
+  // (with kept first positions the walk starts at round 0 and passes over the rounds between them and lo)
+  const int round0 = keep > 0 ? 0 : lo / kWave;
   for (int rd = round0 + (wave - round0 % kWaves + kWaves) % kWaves; rd * kWave <= hi; rd += kWaves) {
     const int c0 = rd * kWave, c = c0 + lane;
-    const bool loaded = c >= lo && c <= hi;
+    if (c0 >= keep && c0 + kWave - 1 < lo) continue;     // (the same for every lane of the wave)
+    const bool loaded = (c >= lo || c < keep) && c <= hi;
     float dot[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) dot[t] = 0.f;
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     // their multiply-adds and keep the plain loops.  The order of every sum is the same.
     constexpr bool BATCHED = HEADS;
     long vbase = -1;
-    if (BATCHED && (lane & 3) == 0 && c <= hi && c + 3 >= lo) {
+    if (BATCHED && (lane & 3) == 0 && c <= hi && (c + 3 >= lo || c < keep)) {
       // the values of four consecutive keys of a dimension are one piece of a page
       const int page = table[c / ps];
       vbase = (long)((size_t)page * v_page_elems + v_head_off + (size_t)((c % ps) >> 2) * 64);
@@ -190,11 +194,11 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
       // a round that holds none of query t's keys leaves its sums as they are
-      const bool takes = c0 <= pos[t] && c0 + kWave - 1 >= first[t];
+      const bool takes = c0 <= pos[t] && (c0 + kWave - 1 >= first[t] || c0 < keep);
       alpha[t] = 1.f;
       p[t] = 0.f;
       if (takes) {
-        const bool valid = c >= first[t] && c <= pos[t];
+        const bool valid = (c >= first[t] || c < keep) && c <= pos[t];
         const float sc = valid ? dot[t] : -INFINITY;
         const float m_new = fmaxf(m[t], wave_max(sc));
         p[t] = valid ? expf(sc - m_new) : 0.f;
@@ -236,7 +240,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 const int key = (quad0 + u) * 4 + e;
-                const bool in = there[u] && c0 + key >= lo && c0 + key <= hi;
+                const bool in = there[u] && (c0 + key >= lo || c0 + key < keep) && c0 + key <= hi;
                 const float v = in ? v4[u][e] : 0.f;   // (the probabilities of such a key are finite: 0 * p adds nothing)
 #pragma unroll
                 for (int t = 0; t < QT; ++t) a[t] = fmaf(p_s[wave][key][t], v, a[t]);
@@ -298,14 +302,14 @@ template <typename T, int SLOTS>
 static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const int* block_tables,
                            const int* positions, const int* req_of_token, GenericItems items,
                            int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int vd, int ps,
-                           int max_pages, float scale, int span, int share_heads, const float* sinks,
+                           int max_pages, float scale, int span, int keep, int share_heads, const float* sinks,
                            hipStream_t stream) {
   const int group = nh / nkv;
 #define TK_ALONE(QT_)                                                                               \
   paged_attention_generic_kernel<T, QT_, true, SLOTS>                                               \
       <<<dim3(num_single, nkv, (group + QT_ - 1) / QT_), kWaves * kWave, 0, stream>>>(              \
           q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd,  \
-          ps, max_pages, scale, span, sinks)
+          ps, max_pages, scale, span, keep, sinks)
   if (num_single > 0) {
     // the heads of a group share a block if that still gives every CU one (the result is the
     // same either way): at batch 64 of an 8B-shaped layer a third faster, at batch 8 slower
@@ -321,7 +325,7 @@ static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const
     paged_attention_generic_kernel<T, kQueries, false, SLOTS>
         <<<dim3(num_tiles, nh, kTileTokens / kQueries), kWaves * kWave, 0, stream>>>(
             q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd, ps,
-            max_pages, scale, span, sinks);
+            max_pages, scale, span, keep, sinks);
 }
 
 // tile_first / tile_count (num_tiles of them) and single (num_single token rows): the step's work
@@ -333,10 +337,11 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
                                       const void* v_cache, const int* block_tables,
                                       const int* positions, const int* req_of_token, void* out,
                                       int N, int nh, int nkv, int hd, int vd, int ps, int max_pages,
-                                      float scale, int span, const int* tile_first,
+                                      float scale, int span, int keep, const int* tile_first,
                                       const int* tile_count, int num_tiles, const int* single,
                                       int num_single, int share_heads, const float* sinks, hipStream_t stream) {
   if (N <= 0) return 0;
+  if (keep < 0 || (keep > 0 && span <= 0)) return -1;
   if (hd > kMaxHd || hd % 8 != 0 || vd > kMaxHd || vd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
   if (tile_first == nullptr) {
     num_tiles = 0;
@@ -349,7 +354,7 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
 #define TK_GENERIC(T_, SLOTS_)                                                                      \
   launch_generic<T_, SLOTS_>((const T_*)q, (const T_*)k_cache, (const T_*)v_cache, block_tables,    \
                              positions, req_of_token, items, num_single, num_tiles, (T_*)out, nh,   \
-                             nkv, hd, vd, ps, max_pages, scale, span, share_heads, sinks, stream)
+                             nkv, hd, vd, ps, max_pages, scale, span, keep, share_heads, sinks, stream)
   if (dtype == 0) {
     if (vd <= 128) TK_GENERIC(float, 2);
     else if (vd <= 256) TK_GENERIC(float, 4);

@@ -15,7 +15,9 @@
 //       (dim, kb) reads the 8 bytes of keys 4 kb .. 4 kb + 3 of its dim), P^T as B: the first product's
 //       result layout is the second's B operand layout.
 // What a token sees besides causality is given by `span`: 0 everything before it, W > 0 the last W
-// positions, -C < 0 the positions of its own chunk of C.  sinks: null, or float32 [nh]: exp(sinks[a])
+// positions, -C < 0 the positions of its own chunk of C; with a window, `keep` > 0 leaves the first
+// `keep` positions of the sequence visible too (their stages of 16 keys are walked first, then the walk
+// jumps to the window's first stage).  sinks: null, or float32 [nh]: exp(sinks[a])
 // is one more term of head a's denominator.
 //
 // Cache pages: K [nkv][hd/8][ps][8], V [nkv][vd/16][ps/4][16][4]; ps a multiple of 16, so that 16
@@ -51,7 +53,7 @@ __global__ __launch_bounds__(kHeadsPerBlock * 64) void attention_tiles_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, const int* __restrict__ tile_first, const int* __restrict__ tile_count,
-    bf16_t* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span,
+    bf16_t* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span, int keep,
     const float* __restrict__ sinks) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
   const int head = blockIdx.y * kHeadsPerBlock + wave;
@@ -83,7 +85,8 @@ __global__ __launch_bounds__(kHeadsPerBlock * 64) void attention_tiles_kernel(
 #pragma unroll
   for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  for (int c0 = lo & ~15; c0 <= hi; c0 += 16) {
+  const int c_first = lo & ~15;
+  for (int c0 = keep > 0 ? 0 : c_first; c0 <= hi; c0 = (c0 + 16 >= keep && c0 + 16 < c_first) ? c_first : c0 + 16) {
     const int page = table[c0 / ps], off = c0 % ps;
     const bf16_t* kp = k_cache + (size_t)page * k_page + k_head + (size_t)(off + col) * 8;
     const bf16_t* vp = v_cache + (size_t)page * v_page + v_head + (size_t)((off >> 2) + kb) * 64 + col * 4;
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(kHeadsPerBlock * 64) void attention_tiles_kernel(
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int key = c0 + kb * 4 + e;
-      seen[e] = key >= first && key <= pos;
+      seen[e] = (key >= first || key < keep) && key <= pos;
       sv[e] = seen[e] ? sc[e] * scale_log2 : -INFINITY;     // (a key that no token wrote may hold anything: chosen, not computed)
     }
     float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(HB * 64) void attention_tiles_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, const int* __restrict__ tile_first, const int* __restrict__ tile_count,
-    bf16_t* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span,
+    bf16_t* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span, int keep,
     const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) bf16_t stage_s[];   // two stages of (hd + vd) * 16 elements
   constexpr int THREADS = HB * 64;
@@ -244,13 +247,15 @@ __global__ __launch_bounds__(HB * 64) void attention_tiles_shared_kernel(
     }                                                                                                          \
   }
   const int c_first = lo & ~15;
-  TK_SFETCH(c_first)
+  const int c_start = keep > 0 ? 0 : c_first;
+  TK_SFETCH(c_start)
   TK_SSTORE(0)
   __syncthreads();
   int buf = 0;
-  for (int c0 = c_first; c0 <= hi; c0 += 16, buf ^= 1) {
-    const bool more = c0 + 16 <= hi;
-    if (more) TK_SFETCH(c0 + 16)
+  for (int c0 = c_start, c_next; c0 <= hi; c0 = c_next, buf ^= 1) {
+    c_next = (c0 + 16 >= keep && c0 + 16 < c_first) ? c_first : c0 + 16;    // (past the kept first positions: on to the window)
+    const bool more = c_next <= hi;
+    if (more) TK_SFETCH(c_next)
     if (computes) {
       const bf16_t* ks = stage_s + (size_t)buf * stage_elems;
       const bf16_t* vs = ks + hd * 16;
@@ -276,7 +281,7 @@ __global__ __launch_bounds__(HB * 64) void attention_tiles_shared_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int key = c0 + kb * 4 + e;
-        seen[e] = key >= first && key <= pos;
+        seen[e] = (key >= first || key < keep) && key <= pos;
         sv[e] = seen[e] ? sc[e] * scale_log2 : -INFINITY;
       }
       float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(HB * 64) void attention_tiles_shared_kernel(
 template <int KCH, int DBL, int HB>
 static int launch_shared(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int max_pages,
                          const int* positions, const int* req_of_token, const int* tile_first, const int* tile_count,
-                         int num_tiles, void* out, int nh, int nkv, int hd, int vd, int ps, float scale, int span,
+                         int num_tiles, void* out, int nh, int nkv, int hd, int vd, int ps, float scale, int span, int keep,
                          const float* sinks, hipStream_t stream) {
   const int group = nh / nkv;
   const size_t lds = (size_t)2 * (hd + vd) * 16 * sizeof(bf16_t);
@@ -359,7 +364,7 @@ static int launch_shared(const void* q, const void* k_cache, const void* v_cache
   if (grid.y > 65535) return -1;
   attention_tiles_shared_kernel<KCH, DBL, HB><<<grid, HB * 64, lds, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions, req_of_token,
-      tile_first, tile_count, (bf16_t*)out, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span, sinks);
+      tile_first, tile_count, (bf16_t*)out, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span, keep, sinks);
   return launch_status();
 }
 
@@ -374,7 +379,8 @@ __global__ __launch_bounds__(256) void attention_heads_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, const int* __restrict__ single, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int nsplit, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span) {
+    float* __restrict__ part_ml, int nsplit, int nh, int nkv, int hd, int vd, int ps, float scale_log2, int span,
+    int keep) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
   const int group = nh / nkv, pieces = (group + 15) >> 4;
   const int kvh = blockIdx.y / pieces, in_group = (blockIdx.y % pieces) * 16 + col;
@@ -402,7 +408,13 @@ __global__ __launch_bounds__(256) void attention_heads_kernel(
 #pragma unroll
   for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  for (int c0 = (first & ~15) + part * 16; c0 <= pos; c0 += parts * 16) {
+  // the stages of the walk in order: those of the kept first positions that lie before the window's first
+  // stage, then the window's; stage s goes to part s % parts
+  const int c_first = first & ~15;
+  const int kept = min((keep + 15) >> 4, c_first >> 4);
+  for (int st = part;; st += parts) {
+    const int c0 = st < kept ? st * 16 : c_first + (st - kept) * 16;
+    if (c0 > pos) break;
     const int page = table[c0 / ps], off = c0 % ps;
     const bf16_t* kp = k_cache + (size_t)page * k_page + k_head + (size_t)(off + col) * 8;
     const bf16_t* vp = v_cache + (size_t)page * v_page + v_head + (size_t)((off >> 2) + kb) * 64 + col * 4;
@@ -427,7 +439,7 @@ __global__ __launch_bounds__(256) void attention_heads_kernel(
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int key = c0 + kb * 4 + e;
-      seen[e] = key >= first && key <= pos;
+      seen[e] = (key >= first || key < keep) && key <= pos;
       sv[e] = seen[e] ? sc[e] * scale_log2 : -INFINITY;
     }
     float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
@@ -527,8 +539,9 @@ __global__ __launch_bounds__(256) void attention_heads_merge_kernel(
 TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                               int max_pages, const int* positions, const int* req_of_token, const int* tile_first,
                               const int* tile_count, int num_tiles, void* out, int nh, int nkv, int hd, int vd, int ps,
-                              float scale, int span, const float* sinks, hipStream_t stream) {
+                              float scale, int span, int keep, const float* sinks, hipStream_t stream) {
   if (num_tiles <= 0) return 0;
+  if (keep < 0 || (keep > 0 && span <= 0)) return -1;
   if (nkv <= 0 || nh % nkv != 0 || hd < 8 || hd % 8 != 0 || vd < 16 || vd % 16 != 0 || ps < 16 || ps % 16 != 0) return -2;
   if (hd > 512 || vd > 512 || (uintptr_t)q % 16 != 0 || (uintptr_t)k_cache % 16 != 0 || (uintptr_t)v_cache % 16 != 0 ||
       (uintptr_t)out % 8 != 0)
@@ -538,7 +551,7 @@ TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_
     // the heads of a kv head share its keys and values through LDS
 #define TK_SHARED(KCH_, DBL_, HB_)                                                                              \
   launch_shared<KCH_, DBL_, HB_>(q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, tile_first, \
-                                 tile_count, num_tiles, out, nh, nkv, hd, vd, ps, scale, span, sinks, stream)
+                                 tile_count, num_tiles, out, nh, nkv, hd, vd, ps, scale, span, keep, sinks, stream)
     if (hd <= 128 && vd <= 128) return group > 4 ? TK_SHARED(4, 8, 8) : TK_SHARED(4, 8, 4);
     if (hd <= 256 && vd <= 256) return group > 4 ? TK_SHARED(8, 16, 8) : TK_SHARED(8, 16, 4);
     return group > 4 ? TK_SHARED(16, 32, 8) : TK_SHARED(16, 32, 4);
@@ -550,7 +563,7 @@ TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_
   attention_tiles_kernel<KCH_, DBL_><<<grid, kHeadsPerBlock * 64, 0, stream>>>(                                \
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,    \
       req_of_token, tile_first, tile_count, (bf16_t*)out, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f,    \
-      span, sinks)
+      span, keep, sinks)
   if (hd <= 128 && vd <= 128) TK_TILES(4, 8);
   else if (hd <= 256 && vd <= 256) TK_TILES(8, 16);
   else TK_TILES(16, 32);
@@ -563,8 +576,10 @@ TK_API int tk_attention_tiles(const void* q, const void* k_cache, const void* v_
 TK_API int tk_attention_heads(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                               int max_pages, const int* positions, const int* req_of_token, const int* single,
                               int num_single, void* out, float* part_o, float* part_ml, int nsplit, int nh, int nkv,
-                              int hd, int vd, int ps, float scale, int span, const float* sinks, hipStream_t stream) {
+                              int hd, int vd, int ps, float scale, int span, int keep, const float* sinks,
+                              hipStream_t stream) {
   if (num_single <= 0) return 0;
+  if (keep < 0 || (keep > 0 && span <= 0)) return -1;
   if (nkv <= 0 || nh % nkv != 0 || hd < 8 || hd % 8 != 0 || vd < 16 || vd % 16 != 0 || ps < 16 || ps % 16 != 0) return -2;
   if (hd > 512 || vd > 512 || (uintptr_t)q % 16 != 0 || (uintptr_t)k_cache % 16 != 0 || (uintptr_t)v_cache % 16 != 0 ||
       (uintptr_t)part_o % 16 != 0 || nsplit < 1 || nsplit > 16 || nh > 65535)    // (the merge: up to 64 parts)
@@ -575,7 +590,7 @@ TK_API int tk_attention_heads(const void* q, const void* k_cache, const void* v_
 #define TK_HEADS(KCH_, DBL_)                                                                                  \
   attention_heads_kernel<KCH_, DBL_><<<grid, 256, 0, stream>>>(                                               \
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,   \
-      req_of_token, single, part_o, part_ml, nsplit, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span)
+      req_of_token, single, part_o, part_ml, nsplit, nh, nkv, hd, vd, ps, scale * 1.4426950408889634f, span, keep)
   if (hd <= 128 && vd <= 128) TK_HEADS(4, 8);
   else if (hd <= 256 && vd <= 256) TK_HEADS(8, 16);
   else TK_HEADS(16, 32);

@@ -545,14 +545,27 @@ __device__ __forceinline__ float gate_act(float z, int act) {
 }
 
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, int act) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, int act,
+                                const float* __restrict__ bias) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t n = idx / I;
   const int i = (int)(idx - n * I);
-  const float g = Elem<T>::load(gu + n * 2 * I + i);
-  const float u = Elem<T>::load(gu + n * 2 * I + I + i);
+  float g = Elem<T>::load(gu + n * 2 * I + i);
+  float u = Elem<T>::load(gu + n * 2 * I + I + i);
+  if (bias) {     // (float32 [2 I]: the gate's biases, then the up projection's)
+    g += bias[i];
+    u += bias[I + i];
+  }
   Elem<T>::store(out + idx, gate_act(g, act) * u);
+}
+
+// x[n, c] += bias[c] in place (float32 bias, the sum formed in float32)
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int H, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  Elem<T>::store(x + idx, Elem<T>::load(x + idx) + bias[idx % H]);
 }
 
 // 8 elements a thread (16-byte loads): I a multiple of 8, pointers 16-byte aligned
@@ -576,11 +589,22 @@ __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __
   *reinterpret_cast<uint4*>(out + n * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, int act, hipStream_t stream) {
+TK_API int tk_add_bias(int dtype, void* x, const float* bias, int N, int H, hipStream_t stream) {
+  if (N <= 0 || H <= 0) return 0;
+  const size_t total = (size_t)N * H;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == 0) add_bias_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, bias, H, total);
+  else add_bias_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, bias, H, total);
+  return launch_status();
+}
+
+// bias: null, or float32 [2 I] added to the gate's and the up projection's halves before the activation
+TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, int act, const float* bias,
+                       hipStream_t stream) {
   if (N <= 0 || I <= 0) return 0;
   if (act != 0 && act != 1) return -1;
   const size_t total = (size_t)N * I;
-  if (dtype == 1 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+  if (bias == nullptr && dtype == 1 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
     const size_t total8 = total / 8;
     silu_mul_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
         (const bf16_t*)gu, (bf16_t*)out, I, total8, act);
@@ -588,9 +612,9 @@ TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, int a
   }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == 0)
-    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total, act);
+    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total, act, bias);
   else
-    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total, act);
+    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total, act, bias);
   return launch_status();
 }
 
@@ -679,18 +703,27 @@ TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long 
 }
 
 // ---------------------------------------------------------------------------
-// Residual add of two parallel branches + norm over rows of width H.
-//   x = resid[row] + (a[row] + b[row]);  if write_resid: resid[row] = x
+// Residual add of up to three parallel branches + norm over rows of width H.
+//   x = resid[row] + scale * (a[row] + b[row] + c[row] + bias);  if write_resid: resid[row] = x
 //   center: out[m] = (x - mean(x)) * rsqrt(mean((x - mean(x))^2) + eps) * weight   (a layer norm without a bias)
 //   else:   out[m] = x * rsqrt(mean(x^2) + eps) * weight
-// A branch is T, float32, or float32 partial sums (added in order); each may be absent.  The
-// two branches' sum is formed first, in float32, and added to the stream once.
+// A branch is T, float32, or float32 partial sums (added in order); each may be absent, and so may
+// the bias (float32 [H], one row for all).  The branches' sum is formed first, in float32, and
+// added to the stream once.  weight2 / out2 (both or neither): the same normalised row times a
+// second weight, for a layer whose two sub-layers each have a norm of their own over the same stream.
 // ---------------------------------------------------------------------------
 struct NormBranch {
   const void* p;
   int f32;
   int parts;
   long stride;
+};
+
+struct NormAdds {
+  NormBranch a, b, c;
+  const float* bias;
+  float scale;
+  __device__ __forceinline__ bool any() const { return a.p || b.p || c.p || bias; }
 };
 
 template <typename T>
@@ -705,25 +738,50 @@ __device__ __forceinline__ float4 branch_four(const NormBranch& b, size_t idx) {
   return s;
 }
 
+// scale * (a + b + c + bias) at four consecutive columns from d of a row that starts at `at`
 template <typename T>
-__device__ __forceinline__ float branches_value(const NormBranch& a, const NormBranch& b, size_t idx) {
-  float s = 0.f;
-  if (a.p) s = branch_value<T>(a.p, a.f32, a.parts, a.stride, idx);
-  if (b.p) s += branch_value<T>(b.p, b.f32, b.parts, b.stride, idx);
+__device__ __forceinline__ float4 adds_four(const NormAdds& n, size_t at, int d) {
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (n.a.p) s = branch_four<T>(n.a, at + d);
+  if (n.b.p) {
+    const float4 t = branch_four<T>(n.b, at + d);
+    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+  }
+  if (n.c.p) {
+    const float4 t = branch_four<T>(n.c, at + d);
+    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+  }
+  if (n.bias) {
+    const float4 t = *reinterpret_cast<const float4*>(n.bias + d);
+    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+  }
+  if (n.scale != 1.f) { s.x *= n.scale; s.y *= n.scale; s.z *= n.scale; s.w *= n.scale; }
   return s;
+}
+
+template <typename T>
+__device__ __forceinline__ float adds_value(const NormAdds& n, size_t at, int d) {
+  float s = 0.f;
+  if (n.a.p) s = branch_value<T>(n.a.p, n.a.f32, n.a.parts, n.a.stride, at + d);
+  if (n.b.p) s += branch_value<T>(n.b.p, n.b.f32, n.b.parts, n.b.stride, at + d);
+  if (n.c.p) s += branch_value<T>(n.c.p, n.c.f32, n.c.parts, n.c.stride, at + d);
+  if (n.bias) s += n.bias[d];
+  return n.scale != 1.f ? s * n.scale : s;
 }
 
 // Vector form: a thread keeps up to kNormGroups pieces of four elements of the row in registers.
 template <typename T>
 __global__ __launch_bounds__(1024) void add_norm2_vec_kernel(
-    float* __restrict__ resid, NormBranch a, NormBranch b, const int* __restrict__ rows,
-    const float* __restrict__ weight, T* __restrict__ out, int H, float eps, int write_resid, int center) {
+    float* __restrict__ resid, NormAdds adds, const int* __restrict__ rows,
+    const float* __restrict__ weight, T* __restrict__ out, const float* __restrict__ weight2, T* __restrict__ out2,
+    int H, float eps, int write_resid, int center) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
   const size_t row = rows ? (size_t)rows[m] : (size_t)m;
   float* x = resid + row * H;
   float4 xv[kNormGroups], wv[kNormGroups];
   float sum = 0.f;
+  const bool adding = adds.any();
 #pragma unroll
   for (int g = 0; g < kNormGroups; ++g) {
     const int d = (g * blockDim.x + threadIdx.x) * 4;
@@ -735,14 +793,8 @@ __global__ __launch_bounds__(1024) void add_norm2_vec_kernel(
     xv[g] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (d < H) {
       float4 v = *reinterpret_cast<const float4*>(x + d);
-      if (a.p || b.p) {
-        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (a.p) s = branch_four<T>(a, row * H + d);
-        if (b.p) {
-          const float4 t = branch_four<T>(b, row * H + d);
-          if (a.p) { s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w; }
-          else s = t;
-        }
+      if (adding) {
+        const float4 s = adds_four<T>(adds, row * H, d);
         v.x += s.x; v.y += s.y; v.z += s.z; v.w += s.w;
         if (write_resid) *reinterpret_cast<float4*>(x + d) = v;
       }
@@ -771,36 +823,42 @@ __global__ __launch_bounds__(1024) void add_norm2_vec_kernel(
       const float4 w = wv[g];
       Store4<T>::at(o + d, make_float4(xv[g].x * rstd * w.x, xv[g].y * rstd * w.y,
                                        xv[g].z * rstd * w.z, xv[g].w * rstd * w.w));
+      if (out2) {
+        const float4 w2 = *reinterpret_cast<const float4*>(weight2 + d);
+        Store4<T>::at(out2 + (size_t)m * H + d, make_float4(xv[g].x * rstd * w2.x, xv[g].y * rstd * w2.y,
+                                                            xv[g].z * rstd * w2.z, xv[g].w * rstd * w2.w));
+      }
     }
   }
 }
 
 // Any width and alignment: the row is walked three times (mean, variance, output).
 template <typename T>
-__global__ void add_norm2_kernel(float* __restrict__ resid, NormBranch a, NormBranch b,
+__global__ void add_norm2_kernel(float* __restrict__ resid, NormAdds adds,
                                  const int* __restrict__ rows, const float* __restrict__ weight,
-                                 T* __restrict__ out, int H, float eps, int write_resid, int center) {
+                                 T* __restrict__ out, const float* __restrict__ weight2, T* __restrict__ out2,
+                                 int H, float eps, int write_resid, int center) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
   const size_t row = rows ? (size_t)rows[m] : (size_t)m;
   float* x = resid + row * H;
-  const bool adds = a.p || b.p;
+  const bool adding = adds.any();
   float sum = 0.f;
   for (int d = threadIdx.x; d < H; d += blockDim.x) {
     float v = x[d];
-    if (adds) {
-      v += branches_value<T>(a, b, row * H + d);
+    if (adding) {
+      v += adds_value<T>(adds, row * H, d);
       if (write_resid) x[d] = v;      // (the passes below then read the sum back)
     }
     sum += v;
   }
-  const bool again = adds && !write_resid;    // the sum is not in the stream: it is formed again
+  const bool again = adding && !write_resid;    // the sum is not in the stream: it is formed again
   float mean = 0.f;
   if (center) mean = block_sum(sum, scratch) / (float)H;
   float ss = 0.f;
   for (int d = threadIdx.x; d < H; d += blockDim.x) {
     float v = x[d];
-    if (again) v += branches_value<T>(a, b, row * H + d);
+    if (again) v += adds_value<T>(adds, row * H, d);
     ss += (v - mean) * (v - mean);
   }
   ss = block_sum(ss, scratch);
@@ -808,30 +866,35 @@ __global__ void add_norm2_kernel(float* __restrict__ resid, NormBranch a, NormBr
   T* o = out + (size_t)m * H;
   for (int d = threadIdx.x; d < H; d += blockDim.x) {
     float v = x[d];
-    if (again) v += branches_value<T>(a, b, row * H + d);
+    if (again) v += adds_value<T>(adds, row * H, d);
     Elem<T>::store(o + d, (v - mean) * rstd * weight[d]);
+    if (out2) Elem<T>::store(out2 + (size_t)m * H + d, (v - mean) * rstd * weight2[d]);
   }
 }
 
 TK_API int tk_add_norm2(int dtype, float* resid, const void* a, int a_f32, int a_parts, long a_stride,
-                        const void* b, int b_f32, int b_parts, long b_stride, const int* rows,
-                        const float* weight, void* out, int M, int H, float eps, int write_resid,
-                        int center, hipStream_t stream) {
+                        const void* b, int b_f32, int b_parts, long b_stride, const void* c, int c_f32, int c_parts,
+                        long c_stride, const float* bias, float scale, const int* rows,
+                        const float* weight, void* out, const float* weight2, void* out2, int M, int H, float eps,
+                        int write_resid, int center, hipStream_t stream) {
   if (M <= 0) return 0;
   if (rows && write_resid) return -1;
-  if (a_parts < 1 || b_parts < 1 || (a_parts > 1 && !a_f32) || (b_parts > 1 && !b_f32)) return -1;
-  const NormBranch ba{a, a_f32 || dtype == 0, a_parts, a_stride}, bb{b, b_f32 || dtype == 0, b_parts, b_stride};
+  if ((weight2 == nullptr) != (out2 == nullptr)) return -1;
+  if (a_parts < 1 || b_parts < 1 || c_parts < 1 || (a_parts > 1 && !a_f32) || (b_parts > 1 && !b_f32) || (c_parts > 1 && !c_f32)) return -1;
+  const NormAdds adds{{a, a_f32 || dtype == 0, a_parts, a_stride}, {b, b_f32 || dtype == 0, b_parts, b_stride},
+                      {c, c_f32 || dtype == 0, c_parts, c_stride}, bias, scale};
   int threads = 64;
   while (threads < 1024 && threads * 4 * (M >= 512 ? kNormGroups : 1) < H) threads *= 2;
-  const bool vec = H % 4 == 0 && H <= threads * 4 * kNormGroups && a_stride % 4 == 0 && b_stride % 4 == 0 &&
+  const bool vec = H % 4 == 0 && H <= threads * 4 * kNormGroups && a_stride % 4 == 0 && b_stride % 4 == 0 && c_stride % 4 == 0 &&
                    ((uintptr_t)resid % 16 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&
-                   ((uintptr_t)weight % 16 == 0) && ((uintptr_t)out % 16 == 0);
+                   ((uintptr_t)c % 16 == 0) && ((uintptr_t)bias % 16 == 0) && ((uintptr_t)weight % 16 == 0) &&
+                   ((uintptr_t)out % 16 == 0) && ((uintptr_t)weight2 % 16 == 0) && ((uintptr_t)out2 % 16 == 0);
   if (vec) {
-    if (dtype == 0) add_norm2_vec_kernel<float><<<M, threads, 0, stream>>>(resid, ba, bb, rows, weight, (float*)out, H, eps, write_resid, center);
-    else add_norm2_vec_kernel<bf16_t><<<M, threads, 0, stream>>>(resid, ba, bb, rows, weight, (bf16_t*)out, H, eps, write_resid, center);
+    if (dtype == 0) add_norm2_vec_kernel<float><<<M, threads, 0, stream>>>(resid, adds, rows, weight, (float*)out, weight2, (float*)out2, H, eps, write_resid, center);
+    else add_norm2_vec_kernel<bf16_t><<<M, threads, 0, stream>>>(resid, adds, rows, weight, (bf16_t*)out, weight2, (bf16_t*)out2, H, eps, write_resid, center);
   } else {
-    if (dtype == 0) add_norm2_kernel<float><<<M, 256, 0, stream>>>(resid, ba, bb, rows, weight, (float*)out, H, eps, write_resid, center);
-    else add_norm2_kernel<bf16_t><<<M, 256, 0, stream>>>(resid, ba, bb, rows, weight, (bf16_t*)out, H, eps, write_resid, center);
+    if (dtype == 0) add_norm2_kernel<float><<<M, 256, 0, stream>>>(resid, adds, rows, weight, (float*)out, weight2, (float*)out2, H, eps, write_resid, center);
+    else add_norm2_kernel<bf16_t><<<M, 256, 0, stream>>>(resid, adds, rows, weight, (bf16_t*)out, weight2, (bf16_t*)out2, H, eps, write_resid, center);
   }
   return launch_status();
 }
@@ -988,6 +1051,7 @@ TK_SLOTS(tk_add_norm2)
 TK_SLOTS(tk_rope_tables)
 TK_SLOTS(tk_qknorm_rope_store)
 TK_SLOTS(tk_silu_mul)
+TK_SLOTS(tk_add_bias)
 TK_SLOTS(tk_scaled_sum)
 TK_SLOTS(tk_rope_norm_store)
 TK_SLOTS(tk_scale_softcap)

@@ -9,6 +9,9 @@
 //     q head a = [dim unrotated | rot_dim rotated]: the unrotated part to q_plain [N, nh, dim], the
 //     rotated part (first `rot` dims rotated, interleaved or half-split pairs) into
 //     q_full[n, a, rank .. rank + rot_dim); channels behind up to the padded key size are zeros;
+//     with q_weight (float32 [dim]) the unrotated part of every q unit is first divided by its root
+//     mean square (eps) and multiplied by q_weight (a query that is itself a normed latent: one unit
+//     of `dim` = its rank); q_full may then be absent;
 //     c = latent / sqrt(mean(latent^2) + eps) * weight (float32 statistics), the key part rotated;
 //     K page [1][hdp/8][ps][8] receives [c | rotated part], V page [1][vdp/16][ps/4][16][4] receives c.
 //   head_linear: out[n, a, m] = sum_k x[n, a, k] W[a, m, k], a product per head, with row and head
@@ -28,7 +31,7 @@ constexpr int kUnitsPerBlock = 4;  // (token, unit) pairs a block, one per wave
 template <typename T, typename TIN>
 __global__ void latent_prepare_kernel(
     const TIN* __restrict__ proj, int parts, long part_stride, const float* __restrict__ c_weight,
-    const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ positions,
+    const float* __restrict__ q_weight, const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, const int* __restrict__ block_tables, T* __restrict__ q_plain,
     T* __restrict__ q_full, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int dim, int rot_dim,
     int rank, int hdp, int vdp, int rot, int interleaved, int ps, int max_pages, float eps, int stores,
@@ -74,7 +77,16 @@ __global__ void latent_prepare_kernel(
   }
   if (is_q) {
     T* qp = q_plain + ((size_t)n * nh + a) * dim;
-    for (int d = lane; d < dim; d += kWave) Elem<T>::store(qp + d, vec[d]);
+    if (q_weight != nullptr) {
+      float qs = 0.f;
+      for (int d = lane; d < dim; d += kWave) qs += vec[d] * vec[d];
+      qs = wave_sum(qs);
+      const float q_rstd = 1.f / sqrtf(qs / (float)dim + eps);
+      for (int d = lane; d < dim; d += kWave) Elem<T>::store(qp + d, vec[d] * q_rstd * q_weight[d]);
+    } else {
+      for (int d = lane; d < dim; d += kWave) Elem<T>::store(qp + d, vec[d]);
+    }
+    if (q_full == nullptr) return;
     T* qf = q_full + ((size_t)n * nh + a) * hdp;
     for (int d = rank + lane; d < hdp; d += kWave) Elem<T>::store(qf + d, d < rank + rot_dim ? vec[dim + d - rank] : 0.f);
     return;
@@ -192,7 +204,8 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
 // proj: [N, nh (dim + rot_dim) (+ rank + rot_dim if stores)] in dtype, or float32 (in_f32; possibly `parts`
 // partial sums, part_stride elements apart).
 TK_API int tk_latent_prepare(int dtype, const void* proj, int in_f32, int parts, long part_stride,
-                             const float* c_weight, const float* cos_t, const float* sin_t, const int* positions,
+                             const float* c_weight, const float* q_weight, const float* cos_t, const float* sin_t,
+                             const int* positions,
                              const int* req_of_token, const int* block_tables, void* q_plain, void* q_full,
                              void* k_cache, void* v_cache, int N, int nh, int dim, int rot_dim, int rank, int hdp,
                              int vdp, int rot, int interleaved, int ps, int max_pages, float eps, int stores,
@@ -204,12 +217,13 @@ TK_API int tk_latent_prepare(int dtype, const void* proj, int in_f32, int parts,
   if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
   if (rot > 0 && (cos_t == nullptr || sin_t == nullptr)) return -1;
   if (stores && (c_weight == nullptr || k_cache == nullptr || v_cache == nullptr)) return -1;
+  if (q_plain == nullptr || (q_full == nullptr && (q_weight == nullptr || rot_dim != 0))) return -1;
   const long units = (long)N * (nh + (stores ? 1 : 0));
   if (units > 0x7fffffffL) return -1;
   const unsigned grid = (unsigned)((units + kUnitsPerBlock - 1) / kUnitsPerBlock);
 #define TK_LP(T_, TIN_)                                                                                   \
   latent_prepare_kernel<T_, TIN_><<<grid, kWave * kUnitsPerBlock, 0, stream>>>(                           \
-      (const TIN_*)proj, parts, part_stride, c_weight, cos_t, sin_t, positions, req_of_token, block_tables, \
+      (const TIN_*)proj, parts, part_stride, c_weight, q_weight, cos_t, sin_t, positions, req_of_token, block_tables, \
       (T_*)q_plain, (T_*)q_full, (T_*)k_cache, (T_*)v_cache, nh, dim, rot_dim, rank, hdp, vdp, rot,       \
       interleaved, ps, max_pages, eps, stores, units)
   if (dtype == 0) TK_LP(float, float);

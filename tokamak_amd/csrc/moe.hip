@@ -54,11 +54,20 @@ template <> struct Vec<bf16_t> {
 
 // A block a token: its waves take the experts two at a time (lanes stride the width), then the
 // first wave picks the largest scores.
+//   correction (null or float32 [E]): the choice is made by score + correction, the weights are the
+//     scores without it.
+//   groups > 0: the experts form `groups` equal groups of neighbours; a group's score is the sum of its
+//     two largest choice scores (of its one, if it has one expert); only experts of the `keep` groups
+//     with the largest scores can be chosen (the others count as minus infinity).
+//   normalise: the chosen experts' weights are divided by their sum (+ 1e-20); then all times `scale`.
 template <typename T>
 __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ chosen,
-    float* __restrict__ weight, int N, int W, int E, int top, int softmax) {
-  extern __shared__ float score[];     // [E]
+    float* __restrict__ weight, int N, int W, int E, int top, int softmax, const float* __restrict__ correction,
+    int groups, int keep, int normalise, float scale) {
+  extern __shared__ float score[];     // [E] scores, [E] choice scores, [groups] group scores
+  float* choice = score + E;
+  float* group_score = choice + E;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int n = blockIdx.x;
   const T* row = h + (size_t)n * W;
@@ -107,12 +116,48 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
     for (int e = lane; e < E; e += kWave) score[e] = expf(score[e] - top_z) / sum;   // (a lane rewrites what it read)
     wave_lds_sync();
   }
-  // the largest `top` scores, one after the other; a lane looks at the experts lane, lane + 64, ...
+  for (int e = lane; e < E; e += kWave) choice[e] = score[e] + (correction ? correction[e] : 0.f);
+  wave_lds_sync();
+  if (groups > 0) {
+    const int size = E / groups;
+    for (int g = lane; g < groups; g += kWave) {
+      float first = -INFINITY, second = -INFINITY;
+      for (int i = 0; i < size; ++i) {
+        const float v = choice[g * size + i];
+        if (v > first) { second = first; first = v; }
+        else if (v > second) second = v;
+      }
+      group_score[g] = size > 1 ? first + second : first;
+    }
+    wave_lds_sync();
+    // the `keep` best groups, one after the other; a kept group's score becomes +infinity
+    for (int k = 0; k < keep; ++k) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += kWave) {
+        const float v = group_score[g];
+        if (v > best && v != INFINITY) { best = v; at = g; }
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) {
+        const float ob = __shfl_xor(best, m, kWave);
+        const int oa = __shfl_xor(at, m, kWave);
+        if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+      }
+      if (lane == 0 && at < groups) group_score[at] = INFINITY;
+      wave_lds_sync();
+    }
+    for (int e = lane; e < E; e += kWave)
+      if (group_score[e / size] != INFINITY) choice[e] = -INFINITY;
+    wave_lds_sync();
+  }
+  // the largest `top` choice scores, one after the other; a lane looks at the experts lane, lane + 64, ...
+  float total = 0.f;      // (lane 0's: the sum of the chosen experts' scores)
   for (int k = 0; k < top; ++k) {
-    float best = -1.f;
+    float best = -INFINITY;
     int at = 0x7fffffff;
     for (int e = lane; e < E; e += kWave) {
-      const float v = score[e];
+      const float v = choice[e];
       if (v > best) { best = v; at = e; }          // (ascending e: the lower index stays on ties)
     }
 #pragma unroll
@@ -121,12 +166,18 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
       const int oa = __shfl_xor(at, m, kWave);
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
+    if (at >= E) at = 0;       // (fewer experts may be chosen than `top`: refused on the host, kept in range here)
     if (lane == 0) {
       chosen[(size_t)n * top + k] = at;
-      weight[(size_t)n * top + k] = best;
-      score[at] = -2.f;
+      weight[(size_t)n * top + k] = score[at];
+      total += score[at];
+      choice[at] = -INFINITY;
     }
     wave_lds_sync();
+  }
+  if (lane == 0 && (normalise || scale != 1.f)) {
+    const float factor = normalise ? scale / (total + 1e-20f) : scale;
+    for (int k = 0; k < top; ++k) weight[(size_t)n * top + k] *= factor;
   }
 }
 
@@ -544,15 +595,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
 // h [N, W] in dtype; router [E, W] float32; chosen [N, top] int32 and weight [N, top] float32 out
 // softmax: the scores are the softmax of the logits over all experts, else their sigmoids
 TK_API int tk_moe_route(int dtype, const void* h, const float* router, int* chosen, float* weight, int N,
-                        int W, int E, int top, int softmax, hipStream_t stream) {
+                        int W, int E, int top, int softmax, const float* correction, int groups, int keep,
+                        int normalise, float scale, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (E < 1 || top < 1 || top > E || W < 1 || (size_t)E * 4 > 64 * 1024) return -1;
+  if (E < 1 || top < 1 || top > E || W < 1 || (size_t)E * 12 > 60 * 1024) return -1;
+  if (groups < 0 || (groups > 0 && (E % groups != 0 || keep < 1 || keep > groups || (long)keep * (E / groups) < top))) return -1;
   const unsigned blocks = (unsigned)N;
-  const size_t lds = (size_t)E * sizeof(float);
+  const size_t lds = ((size_t)2 * E + (size_t)groups) * sizeof(float);
   if (dtype == 0)
-    moe_route_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>((const float*)h, router, chosen, weight, N, W, E, top, softmax);
+    moe_route_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>((const float*)h, router, chosen, weight, N, W, E, top, softmax,
+                                                                         correction, groups, keep, normalise, scale);
   else
-    moe_route_kernel<bf16_t><<<blocks, kRouteWaves * kWave, lds, stream>>>((const bf16_t*)h, router, chosen, weight, N, W, E, top, softmax);
+    moe_route_kernel<bf16_t><<<blocks, kRouteWaves * kWave, lds, stream>>>((const bf16_t*)h, router, chosen, weight, N, W, E, top, softmax,
+                                                                          correction, groups, keep, normalise, scale);
   return launch_status();
 }
 

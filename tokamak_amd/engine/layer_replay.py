@@ -150,6 +150,9 @@ class LayerRecording:
     result: object
     packed: PackedCalls | None = field(default=None, repr=False)
     pack_tried: bool = field(default=False, repr=False)
+    # fields of the result that are tensors of the layer itself (a bias that its last product leaves to
+    # the residual add): (field, tensor key); a replayed layer hands on its own
+    result_own: tuple = ()
 
     def launch(self, tensors: dict[tuple, torch.Tensor], then):
         if self.packed is not None:
@@ -169,6 +172,8 @@ class LayerRecording:
                 packed = PackedCalls(self.calls)
                 self.packed = packed if packed.ok else None
         result = self.result
+        if self.result_own:
+            result = dataclasses.replace(result, **{name: tensors[key] for name, key in self.result_own})
         if isinstance(result, Added) and result.gamma is not None:
             # the stream times the weight of the norm that follows THIS layer
             result = dataclasses.replace(result, gamma=then.sink(None).gamma)
@@ -194,4 +199,9 @@ def record(run, tensors: dict[tuple, torch.Tensor]):
             if at >= 0 and spans[at][0] <= arg.value < spans[at][1]:
                 patches.append((index, spans[at][2], arg.value - spans[at][0]))
         calls.append((fn, args, tuple(patches), status))
-    return result, LayerRecording(calls, recorder.keep, result)
+    result_own = ()
+    if dataclasses.is_dataclass(result):
+        by_address = {(t.data_ptr(), tuple(t.shape)): key for key, t in tensors.items() if key[0] == "part" and t.numel()}
+        result_own = tuple((name, by_address[(t.data_ptr(), tuple(t.shape))]) for name, t in _fields(result)
+                           if (t.data_ptr(), tuple(t.shape)) in by_address)
+    return result, LayerRecording(calls, recorder.keep, result, result_own=result_own)

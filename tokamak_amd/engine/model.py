@@ -148,20 +148,21 @@ class LayeredModel:
                 if slot in requests and requests[slot] != req:
                     raise ValueError(f"cache slot {slot} is written with two different layouts")
                 requests[slot] = req
-        windows: list[int | None] = []
+        # a retention rule: (window, kept first positions)
+        rules: list[tuple[int | None, int]] = []
         for req in requests.values():
-            if req.window not in windows:
-                windows.append(req.window)
-        windows.sort(key=lambda w: (w is not None, w or 0))
+            if (req.window, req.keep_first) not in rules:
+                rules.append((req.window, req.keep_first))
+        rules.sort(key=lambda r: (r[0] is not None, r[0] or 0, r[1]))
         groups = [
             CacheGroupSpec(
-                name="full" if w is None else f"window{w}",
-                slots=tuple(s for s, r in sorted(requests.items()) if r.window == w),
-                window=w,
+                name="full" if w is None else f"window{w}" + (f"+first{k}" if k else ""),
+                slots=tuple(s for s, r in sorted(requests.items()) if (r.window, r.keep_first) == (w, k)),
+                window=w, keep_first=k,
             )
-            for w in windows
+            for w, k in rules
         ]
-        slots = {s: SlotLayout(windows.index(r.window), r) for s, r in requests.items()}
+        slots = {s: SlotLayout(rules.index((r.window, r.keep_first)), r) for s, r in requests.items()}
         return groups, slots
 
     def state_requests(self) -> dict[int, dict[str, StateArray]]:

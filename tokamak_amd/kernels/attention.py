@@ -288,7 +288,8 @@ def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, 
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads, num_kv_heads,
-                    head_dim, page_size, scale, window=None, value_dim=None, chunk=None, sinks=None) -> None:
+                    head_dim, page_size, scale, window=None, value_dim=None, chunk=None, sinks=None,
+                    keep_first=0) -> None:
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages
     of each token's request.
 
@@ -304,7 +305,8 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     matrix cores where the shape fits (tiles of 16, walking from the chunk's first stage),
     single tokens (which read a chunk at most) and everything else in the generic kernel.
     ``sinks``: float32 [num_heads], one more term exp(sinks[a]) of head a's denominator, added where
-    a row's sums are complete (every kernel has it).
+    a row's sums are complete (every kernel has it).  ``keep_first``: with a window, the first so many
+    positions of a sequence stay visible (the window kernels take it).
     bfloat16 at other shapes (key and value sizes that differ or are not 64 or 128, a window), with pages
     of a multiple of 16 tokens: the portions' tiles on the matrix cores with operands straight from the
     pages, or through LDS for the heads of one kv head (``ops.attention_tiles``); tokens that run alone
@@ -363,7 +365,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             if not ops.attention_tiles(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.tile_first,
                                        work.tile_count, work.num_tiles, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
                                        head_dim=head_dim, value_dim=value_dim, page_size=page_size, scale=scale, window=window,
-                                       chunk=chunk, sinks=sinks):
+                                       chunk=chunk, sinks=sinks, keep_first=keep_first):
                 raise ops.KernelError("the tile kernel refused a shape it was asked about")
         if profiling and work.num_single:
             ops._note(f"{work.num_single} tokens {head_dim}/{value_dim}", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
@@ -371,12 +373,15 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             ops.attention_heads(q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, work.single,
                                 work.num_single, out, num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
                                 value_dim=value_dim, page_size=page_size, scale=scale, window=window, chunk=chunk, sinks=sinks,
-                                num_splits=heads_form_splits(work.num_single, num_kv_heads, group, work.max_single_len, window, chunk))
+                                keep_first=keep_first,
+                                num_splits=heads_form_splits(work.num_single, num_kv_heads, group, work.max_single_len,
+                                                             window + keep_first if window else window, chunk))
         elif work.num_single:
             ops.paged_attention_generic(
                 q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
                 num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-                scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks)
+                scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True, sinks=sinks,
+                keep_first=keep_first)
         return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
@@ -384,7 +389,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-        scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, sinks=sinks)
+        scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles, sinks=sinks, keep_first=keep_first)
 
 
 def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *, num_heads, num_kv_heads,

@@ -170,8 +170,9 @@ _SIGS = {
         "tk_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p,
                            c_void_p, c_int, c_int, c_float, c_int, c_void_p],
-        "tk_add_norm2": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p,
-                         c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_int, c_void_p],
+        "tk_add_norm2": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long,
+                         c_void_p, c_int, c_int, c_long, c_void_p, c_float, c_void_p,
+                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_int, c_void_p],
         "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
         "tk_qknorm_rope_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -181,7 +182,8 @@ _SIGS = {
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                c_int, c_void_p, c_int, c_void_p, c_void_p],
         "tk_scale_softcap": [c_void_p, c_long, c_float, c_float, c_void_p],
-        "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+        "tk_add_bias": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "tk_scaled_sum": [c_int, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float,
                           c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
@@ -216,7 +218,8 @@ _SIGS = {
                         c_float, c_float, c_float, c_void_p],
     },
     "moe": {
-        "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                         c_int, c_int, c_int, c_float, c_void_p],
         "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_void_p],
         "tk_moe_down": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -252,11 +255,11 @@ _SIGS = {
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p,
+                                       c_float, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p,
                                        c_void_p],
     },
     "latent": {
-        "tk_latent_prepare": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        "tk_latent_prepare": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
         "tk_head_linear": [c_int, c_void_p, c_long, c_long, c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int,
@@ -269,10 +272,18 @@ _SIGS = {
     },
     "attention_tiles": {
         "tk_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                               c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
+                               c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
         "tk_attention_heads": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                c_void_p, c_void_p],
+    },
+    "ssm": {
+        "tk_conv_silu": [c_int, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_ssd_scan": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_gated_group_norm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p,
+                                c_int, c_int, c_int, c_float, c_void_p],
     },
     "attention_fused": {
         "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -440,16 +451,25 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
 
 
 def add_norm2(resid: torch.Tensor, a: torch.Tensor | None, b: torch.Tensor | None, weight: torch.Tensor, eps: float,
-              out: torch.Tensor, *, center: bool, rows: torch.Tensor | None = None, write_resid: bool = True) -> None:
-    """x = resid[row] + (a[row] + b[row]), optionally stored back; ``center``: out = (x - mean) /
-    sqrt(mean((x - mean)^2) + eps) * weight (a layer norm without a bias), else the RMS norm.  ``a`` and
-    ``b`` are each None, [M, H] in the compute dtype or float32, or float32 partial sums [P, M, H]."""
-    _gpu(resid, a, b, weight, out, rows)
+              out: torch.Tensor, *, center: bool, rows: torch.Tensor | None = None, write_resid: bool = True,
+              c: torch.Tensor | None = None, bias: torch.Tensor | None = None, scale: float = 1.0,
+              weight2: torch.Tensor | None = None, out2: torch.Tensor | None = None) -> None:
+    """x = resid[row] + scale * (a[row] + b[row] + c[row] + bias), optionally stored back; ``center``: out =
+    (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight (a layer norm without a bias), else the RMS norm.
+    ``a``, ``b`` and ``c`` are each None, [M, H] in the compute dtype or float32, or float32 partial sums
+    [P, M, H]; ``bias`` is None or float32 [H].  ``weight2`` and ``out2`` (both or neither): the same normalised
+    row times a second weight, for two sub-layers that each norm the same stream."""
+    _gpu(resid, a, b, c, bias, weight, out, rows, weight2, out2)
     h = resid.shape[-1]
     m = out.shape[0] if rows is None else rows.numel()
     _need(resid.dtype == torch.float32 and weight.dtype == torch.float32, "residual and norm weight are float32")
     _need(weight.numel() == h and out.shape[-1] == h and out.shape[0] >= m, "norm shapes disagree")
-    adds = a is not None or b is not None
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == h), "the bias is float32 [H]")
+    _need((weight2 is None) == (out2 is None), "a second weight and a second output come together")
+    if weight2 is not None:
+        _need(weight2.dtype == torch.float32 and weight2.numel() == h and out2.dtype == out.dtype
+              and out2.shape[-1] == h and out2.shape[0] >= m, "the second norm's shapes disagree")
+    adds = a is not None or b is not None or c is not None or bias is not None
     if rows is None:
         _need(resid.shape[0] >= m, "residual has fewer rows than the output")
     else:
@@ -457,11 +477,13 @@ def add_norm2(resid: torch.Tensor, a: torch.Tensor | None, b: torch.Tensor | Non
         write_resid = False
     pa, fa, na, sa = _branch(a, resid.shape[0], h, out.dtype, "a")
     pb, fb, nb, sb = _branch(b, resid.shape[0], h, out.dtype, "b")
-    _note(f"{m}x{h}", m * h * (4 + (8 if write_resid and adds else 0) + out.element_size())
-          + sum(t.element_size() * parts * m * h for t, parts in ((a, na), (b, nb)) if t is not None))
-    _check(_fn("elementwise", "tk_add_norm2")(_code(out.dtype), _p(resid), pa, fa, na, sa, pb, fb, nb, sb, _p(rows),
-                                              _p(weight), _p(out), m, h, float(eps), int(bool(write_resid)),
-                                              int(bool(center)), _stream()), "add_norm2")
+    pc, fc, nc, sc = _branch(c, resid.shape[0], h, out.dtype, "c")
+    _note(f"{m}x{h}", m * h * (4 + (8 if write_resid and adds else 0) + out.element_size() * (2 if out2 is not None else 1))
+          + sum(t.element_size() * parts * m * h for t, parts in ((a, na), (b, nb), (c, nc)) if t is not None))
+    _check(_fn("elementwise", "tk_add_norm2")(_code(out.dtype), _p(resid), pa, fa, na, sa, pb, fb, nb, sb, pc, fc, nc, sc,
+                                              _p(bias), float(scale), _p(rows), _p(weight), _p(out), _p(weight2), _p(out2),
+                                              m, h, float(eps), int(bool(write_resid)), int(bool(center)), _stream()),
+           "add_norm2")
 
 
 def rope_tables(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor,
@@ -590,15 +612,26 @@ def scale_softcap(logits: torch.Tensor, scale: float, cap: float | None) -> None
 GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
-    """out[n, i] = act(gate_up[n, i]) * gate_up[n, I + i]; act is silu, or the tanh form of gelu."""
-    _gpu(gate_up, out)
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu", bias: torch.Tensor | None = None) -> None:
+    """out[n, i] = act(gate_up[n, i]) * gate_up[n, I + i]; act is silu, or the tanh form of gelu.  ``bias``:
+    float32 [2 I], added to both halves before the activation."""
+    _gpu(gate_up, out, bias)
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == gate_up.shape[1]), "the bias is float32 [2 I]")
     n, two_i = gate_up.shape
     _need(two_i % 2 == 0 and out.shape == (n, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes disagree")
     _note(f"{n}x{two_i // 2}", n * two_i * out.element_size() * 1.5)
     _need(activation in GATE_ACTIVATIONS, f"the gate's activation is one of {sorted(GATE_ACTIVATIONS)}")
     _check(_fn("elementwise", "tk_silu_mul")(_code(out.dtype), _p(gate_up), _p(out), n, two_i // 2,
-                                             GATE_ACTIVATIONS[activation], _stream()), "silu_mul")
+                                             GATE_ACTIVATIONS[activation], _p(bias), _stream()), "silu_mul")
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """x[n, c] += bias[c] in place; x [N, H] in the compute dtype or float32, bias float32 [H]."""
+    _gpu(x, bias)
+    n, h = x.shape
+    _need(bias.dtype == torch.float32 and bias.numel() == h, "the bias is float32 [H]")
+    _note(f"{n}x{h}", 2 * n * h * x.element_size())
+    _check(_fn("elementwise", "tk_add_bias")(_code(x.dtype), _p(x), _p(bias), n, h, _stream()), "add_bias")
 
 
 def _branch(t: torch.Tensor | None, rows: int, width: int, dtype: torch.dtype, what: str):
@@ -898,23 +931,125 @@ def gla_column_splits(requests: int, heads: int, vdim: int, longest: int) -> int
     return splits
 
 
+SSM_MAX_TAPS = 8             # taps of the short convolution (csrc/ssm.hip: kMaxTaps)
+SSM_SPLIT_FROM_TOKENS = 64   # a request's tokens in a step from which a head's value columns are shared out
+SSM_SPLIT_MIN_COLUMNS = 8
+SSM_SPLIT_BLOCKS = 1024
+
+
+def _ssm_in(t: torch.Tensor, rows: int, dtype: torch.dtype, what: str):
+    """(pointer, is_f32, parts, part_stride, row length) of a projection [rows, ld] in ``dtype`` or float32, or of
+    float32 partial sums [parts, rows, ld]."""
+    ld = t.shape[-1]
+    pointer, is_f32, parts, stride = _branch(t, rows, ld, dtype, what)
+    return pointer, is_f32, parts, stride, ld
+
+
+def conv_silu(proj: torch.Tensor, col0: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor | None,
+              out: torch.Tensor, batch) -> None:
+    """out[t, c] = silu(bias[c] + sum_j weight[c, j] x_(t - (taps - 1) + j)[c]) with x the columns col0 .. col0 + C of
+    ``proj`` ([N, ld] in out's dtype or float32, or float32 partial sums [P, N, ld]): a causal convolution per
+    channel whose last tap meets the token itself.  The inputs before a step's first token come from ``state``
+    (float32 [slots, taps - 1, C], oldest first; zeros before a sequence's start), which then takes the step's last
+    inputs.  weight float32 [C, taps], bias float32 [C]."""
+    _gpu(proj, weight, bias, state, out)
+    n, c = out.shape
+    taps = weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (c, taps) and bias.dtype == torch.float32 and bias.numel() == c,
+          "the convolution's weight is float32 [channels, taps], its bias float32 [channels]")
+    _need(1 <= taps <= SSM_MAX_TAPS, f"the convolution has 1 to {SSM_MAX_TAPS} taps")
+    _need(taps == 1 or (state is not None and state.dtype == torch.float32 and tuple(state.shape[1:]) == (taps - 1, c)),
+          "the convolution's state is float32 [slots, taps - 1, channels]")
+    _need(batch.num_tokens == n, "the step's descriptor does not match")
+    pointer, is_f32, parts, stride, ld = _ssm_in(proj, n, out.dtype, "projections")
+    _need(0 <= col0 and col0 + c <= ld, "the convolution's channels lie outside the projections")
+    _note(f"{n}x{c}x{taps}", n * c * (proj.element_size() * parts + out.element_size()))
+    _check(_fn("ssm", "tk_conv_silu")(_code(out.dtype), pointer, is_f32, parts, stride, ld, int(col0), _p(weight), _p(bias),
+                                      _p(state), _p(batch.q_start), _p(batch.state_slots), _p(out), batch.num_requests,
+                                      c, taps, batch.max_q_len, _stream()), "conv_silu")
+
+
+def ssd_column_splits(requests: int, heads: int, vdim: int, longest: int) -> int:
+    """Blocks that share a head's value columns in the scan: one in steps of few tokens a request; in a long
+    portion as many as give some 1,024 blocks, each with 8 columns or more (the columns never meet)."""
+    if longest < SSM_SPLIT_FROM_TOKENS:
+        return 1
+    splits = 1
+    while (requests * heads * splits < SSM_SPLIT_BLOCKS and vdim // (2 * splits) >= SSM_SPLIT_MIN_COLUMNS
+           and vdim % (2 * splits) == 0):
+        splits *= 2
+    return splits
+
+
+def ssd_scan(u: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
+             skip: torch.Tensor, state: torch.Tensor, y: torch.Tensor, batch, *, heads: int, groups: int, state_size: int,
+             vdim: int) -> None:
+    """Per request and head over the step's tokens in order: dt = softplus(proj[t, dt_col + head] + dt_bias),
+    S <- exp(-exp(a_log) dt) S + dt B_t x_t^T, y_t = S^T C_t + skip x_t, with x, B, C the columns of ``u``
+    ([N, heads * vdim + 2 groups * state_size], the convolution's output; head h reads group h // (heads / groups)),
+    S float32 [slots, heads, state_size, vdim] (kept) and y float32 [N, heads * vdim]."""
+    _gpu(u, proj, dt_bias, a_log, skip, state, y)
+    n = y.shape[0]
+    c = heads * vdim + 2 * groups * state_size
+    _need(heads % groups == 0 and u.shape == (n, c) and y.dtype == torch.float32 and y.shape == (n, heads * vdim),
+          "the scan's operands do not match its sizes")
+    _need(all(t.dtype == torch.float32 and t.numel() == heads for t in (dt_bias, a_log, skip)), "a head's constants are float32 [heads]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, state_size, vdim),
+          "the state is float32 [slots, heads, state, vdim]")
+    _need(1 <= vdim <= 1024 and 1 <= state_size <= 1024 and batch.num_tokens == n, "the scan takes sizes up to 1,024")
+    pointer, is_f32, parts, stride, ld = _ssm_in(proj, n, u.dtype, "projections")
+    _need(0 <= dt_col and dt_col + heads <= ld, "the step sizes lie outside the projections")
+    splits = ssd_column_splits(batch.num_requests, heads, vdim, batch.max_q_len)
+    _note(f"{n}x{heads}x{state_size}x{vdim}", n * (c * u.element_size() + heads * vdim * 4), 6.0 * n * heads * state_size * vdim)
+    _check(_fn("ssm", "tk_ssd_scan")(_code(u.dtype), _p(u), pointer, is_f32, parts, stride, ld, int(dt_col), _p(dt_bias),
+                                     _p(a_log), _p(skip), _p(state), _p(batch.q_start), _p(batch.state_slots), _p(y),
+                                     batch.num_requests, heads, groups, state_size, vdim, splits, _stream()), "ssd_scan")
+
+
+def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, weight: torch.Tensor, out: torch.Tensor, *,
+                     groups: int, eps: float) -> None:
+    """g = y * silu(z) with z the columns z_col .. z_col + inner of ``proj``; out = g / rms(g) * weight, the root
+    mean square taken over each of ``groups`` equal parts of the row.  y float32 [N, inner], weight float32 [inner]."""
+    _gpu(y, proj, weight, out)
+    n, inner = out.shape
+    _need(y.dtype == torch.float32 and y.shape == (n, inner) and weight.dtype == torch.float32 and weight.numel() == inner
+          and groups >= 1 and inner % groups == 0, "the gated norm's operands do not match")
+    pointer, is_f32, parts, stride, ld = _ssm_in(proj, n, out.dtype, "projections")
+    _need(0 <= z_col and z_col + inner <= ld, "the gate lies outside the projections")
+    _note(f"{n}x{inner}/{groups}", n * inner * (4 + proj.element_size() * parts + out.element_size()))
+    _check(_fn("ssm", "tk_gated_group_norm")(_code(out.dtype), _p(y), pointer, is_f32, parts, stride, ld, int(z_col),
+                                             _p(weight), _p(out), n, inner, groups, float(eps), _stream()), "gated_group_norm")
+
+
 MOE_LDS_BYTES = 96 * 1024      # of a row of activations in float32 that a block of the expert kernels stages
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, top: int,
-              scoring: str = "sigmoid") -> None:
+              scoring: str = "sigmoid", *, correction: torch.Tensor | None = None, groups: tuple[int, int] | None = None,
+              normalise: bool = False, scale: float = 1.0) -> None:
     """Per token the ``top`` experts with the largest scores, float32 throughout: the scores are
     sigmoid(router . h), or with ``scoring="softmax"`` the softmax of router . h over all experts;
-    chosen [N, top] int32 (largest first, the lower index on ties), weight [N, top] float32 their scores."""
+    chosen [N, top] int32 (largest first, the lower index on ties), weight [N, top] float32 their scores.
+    ``correction`` (float32 [experts]): the choice goes by score + correction, the weights stay the scores.
+    ``groups`` = (count, keep): the experts form ``count`` equal groups of neighbours, a group's score is the
+    sum of its two largest choice scores, and only experts of the ``keep`` best groups can be chosen.
+    ``normalise``: the chosen weights are divided by their sum (+ 1e-20); then all are multiplied by ``scale``."""
     _need(scoring in ("sigmoid", "softmax"), "the router's scores are sigmoids or a softmax")
-    _gpu(h, router, chosen, weight)
+    _gpu(h, router, chosen, weight, correction)
     n, w = h.shape
     e = router.shape[0]
     _need(router.dtype == torch.float32 and router.shape == (e, w), "the router is float32 [experts, width]")
     _need(1 <= top <= e and chosen.dtype == torch.int32 and weight.dtype == torch.float32
           and chosen.numel() >= n * top and weight.numel() >= n * top, "lists of chosen experts too small")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == e),
+          "the correction is float32 [experts]")
+    count, keep = groups or (0, 0)
+    if groups:
+        _need(count >= 1 and e % count == 0 and 1 <= keep <= count and keep * (e // count) >= top,
+              "groups divide the experts evenly and the kept ones hold at least `top` experts")
     _check(_fn("moe", "tk_moe_route")(_code(h.dtype), _p(h), _p(router), _p(chosen), _p(weight), n, w, e, top,
-                                      int(scoring == "softmax"), _stream()), "moe_route")
+                                      int(scoring == "softmax"), _p(correction), int(count), int(keep),
+                                      int(bool(normalise)), float(scale), _stream()), "moe_route")
 
 
 def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, act: torch.Tensor,
@@ -1336,22 +1471,29 @@ def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor | None, cos: 
                    block_tables: torch.Tensor, q_plain: torch.Tensor, q_full: torch.Tensor,
                    k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int, head_dim: int,
                    rot_dim: int, rank: int, rotary_dim: int, interleaved: bool, page_size: int, eps: float,
-                   store: bool = True) -> None:
+                   store: bool = True, q_weight: torch.Tensor | None = None) -> None:
     """From a token's projections [q heads of (head_dim unrotated | rot_dim rotated) | latent of ``rank`` |
     one key part of rot_dim] (the last two only with ``store``): the unrotated query parts to q_plain
     [N, heads, head_dim]; the rotated ones into q_full[n, a, rank : rank + rot_dim] (q_full is [N, heads,
     padded key size]; its first ``rank`` channels are left for the query carried into the latent's space);
     the latent divided by its root mean square (``eps``) times ``latent_weight`` and the rotated key part
-    into the K page as one key [latent | rotated part], the latent also into the V page."""
-    _gpu(proj, latent_weight, cos, sin, positions, req_of_token, block_tables, q_plain, q_full, k_cache, v_cache)
+    into the K page as one key [latent | rotated part], the latent also into the V page.  ``q_weight``
+    (float32 [head_dim]): the unrotated part of every query unit is divided by its root mean square (``eps``)
+    and multiplied by it first (a query that is itself a normed latent); ``q_full`` may then be None if
+    nothing is rotated."""
+    _gpu(proj, latent_weight, cos, sin, positions, req_of_token, block_tables, q_plain, q_full, k_cache, v_cache, q_weight)
+    _need(q_weight is None or (q_weight.dtype == torch.float32 and q_weight.numel() == head_dim),
+          "the query norm's weight is float32 [head_dim]")
+    _need(q_full is not None or (q_weight is not None and rot_dim == 0), "q_full may be absent only for a normed, unrotated query")
     n = positions.numel()
     qw = head_dim + rot_dim
     width = num_heads * qw + (rank + rot_dim if store else 0)
-    in_f32, parts, stride = _partials(proj, n, width, q_full.dtype, "projections")
+    in_f32, parts, stride = _partials(proj, n, width, q_plain.dtype, "projections")
     hdp, vdp = padded_sizes(rank + rot_dim, rank)
     _need(max(qw, rank + rot_dim) <= 1024 and max(hdp, vdp) <= 512, "heads of up to 1,024 and keys of up to 512 channels")
-    _need(q_plain.dtype == q_full.dtype and q_plain.numel() >= n * num_heads * head_dim
-          and q_full.numel() >= n * num_heads * hdp, "q_plain / q_full too small")
+    _need(q_plain.numel() >= n * num_heads * head_dim
+          and (q_full is None or (q_plain.dtype == q_full.dtype and q_full.numel() >= n * num_heads * hdp)),
+          "q_plain / q_full too small")
     _need(rotary_dim % 2 == 0 and 0 <= rotary_dim <= rot_dim and page_size % 8 == 0, "rotary_dim is even and at most rot_dim")
     _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32
                                and sin.dtype == torch.float32 and cos.numel() >= n * (rotary_dim // 2)
@@ -1361,12 +1503,12 @@ def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor | None, cos: 
     if store:
         _need(latent_weight is not None and latent_weight.dtype == torch.float32 and latent_weight.numel() == rank,
               "the latent's norm weight is float32 [rank]")
-        _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_full.dtype == v_cache.dtype
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_plain.dtype == v_cache.dtype
               and k_cache.numel() % (hdp * page_size) == 0 and v_cache.numel() % (vdp * page_size) == 0
               and k_cache.numel() // hdp == v_cache.numel() // vdp, "cache size is not whole pages")
-    _note(f"{n}x{width}", n * width * (proj.element_size() * parts + q_full.element_size()))
+    _note(f"{n}x{width}", n * width * (proj.element_size() * parts + q_plain.element_size()))
     _check(_fn("latent", "tk_latent_prepare")(
-        _code(q_full.dtype), _p(proj), in_f32, parts, stride, _p(latent_weight), _p(cos), _p(sin), _p(positions),
+        _code(q_plain.dtype), _p(proj), in_f32, parts, stride, _p(latent_weight), _p(q_weight), _p(cos), _p(sin), _p(positions),
         _p(req_of_token), _p(block_tables), _p(q_plain), _p(q_full), _p(k_cache if store else None),
         _p(v_cache if store else None), n, num_heads, head_dim, rot_dim, rank, hdp, vdp, rotary_dim,
         int(bool(interleaved)), page_size, block_tables.shape[1], float(eps), int(bool(store)), _stream()), "latent_prepare")
@@ -1395,7 +1537,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             window: int | None = None, tiles: tuple | None = None,
                             share_heads: bool | None = None, value_dim: int | None = None,
                             chunk: int | None = None, only_single: bool = False,
-                            sinks: torch.Tensor | None = None) -> None:
+                            sinks: torch.Tensor | None = None, keep_first: int = 0) -> None:
     """Causal attention of each query token over its request's pages.  ``tiles``:
     (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
     of up to 16 consecutive tokens of one request, and token rows that run alone), which together
@@ -1406,8 +1548,10 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     ``head_dim``.  ``chunk``: a query sees only the keys of its own chunk of that many positions
     (counted from position 0); not together with ``window``.  ``only_single``: the tokens of the tiles
     are left to another kernel.  ``sinks``: float32 [num_heads]; head a's softmax has exp(sinks[a]) as one
-    more term of its denominator, with no key and no value."""
+    more term of its denominator, with no key and no value.  ``keep_first``: with a window, the first so many
+    positions of a sequence stay visible whatever the distance."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out, sinks)
+    _need(keep_first >= 0 and (keep_first == 0 or window), "kept first positions go with a window")
     _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads), "sinks are float32 [num_heads]")
     n = positions.numel()
     vd = head_dim if value_dim is None else int(value_dim)
@@ -1442,7 +1586,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _check(_fn("attention_generic", "tk_paged_attention_generic")(
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
         _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, vd, page_size,
-        block_tables.shape[1], float(scale), span, _p(tile_first), _p(tile_count), num_tiles,
+        block_tables.shape[1], float(scale), span, int(keep_first), _p(tile_first), _p(tile_count), num_tiles,
         _p(single), num_single, -1 if share_heads is None else int(share_heads), _p(sinks), _stream()),
         "paged_attention_generic")
 
@@ -1454,7 +1598,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     positions: torch.Tensor, req_of_token: torch.Tensor, tile_first: torch.Tensor,
                     tile_count: torch.Tensor, num_tiles: int, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, value_dim: int, page_size: int, scale: float, window: int | None = None,
-                    chunk: int | None = None, sinks: torch.Tensor | None = None) -> bool:
+                    chunk: int | None = None, sinks: torch.Tensor | None = None, keep_first: int = 0) -> bool:
     """bf16 attention of the tiles of prompt portions (up to 16 consecutive tokens of one request each) on
     the matrix cores, for keys and values of unlike sizes (up to 512; keys in pieces of 8, values in blocks
     of 16), any group, a window or chunks, sinks; pages of a multiple of 16 tokens.  Returns False
@@ -1477,7 +1621,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     status = _fn("attention_tiles", "tk_attention_tiles")(
         _p(q), _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(positions), _p(req_of_token),
         _p(tile_first), _p(tile_count), num_tiles, _p(out), num_heads, num_kv_heads, head_dim, value_dim, page_size,
-        float(scale), span, _p(sinks), _stream())
+        float(scale), span, int(keep_first if window else 0), _p(sinks), _stream())
     if status == NOT_INSTANTIATED:
         return False
     _check(status, "attention_tiles")
@@ -1552,7 +1696,7 @@ def attention_heads(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     positions: torch.Tensor, req_of_token: torch.Tensor, single: torch.Tensor, num_single: int,
                     out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
                     page_size: int, scale: float, num_splits: int, window: int | None = None,
-                    chunk: int | None = None, sinks: torch.Tensor | None = None) -> None:
+                    chunk: int | None = None, sinks: torch.Tensor | None = None, keep_first: int = 0) -> None:
     """bf16 attention of tokens that run alone (``single``: their rows) on the matrix cores, the 16 columns of
     a product being 16 query heads of one kv head, for the shapes of ``attention_tiles``.  Each token's visible
     keys are dealt, 16 at a time, to the four waves of ``num_splits`` blocks; a second kernel merges the waves'
@@ -1577,7 +1721,7 @@ def attention_heads(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _check(_fn("attention_tiles", "tk_attention_heads")(
         _p(q), _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(positions), _p(req_of_token),
         _p(single), num_single, _p(out), _p(part_o), _p(part_ml), num_splits, num_heads, num_kv_heads, head_dim,
-        value_dim, page_size, float(scale), span, _p(sinks), _stream()), "attention_heads")
+        value_dim, page_size, float(scale), span, int(keep_first if window else 0), _p(sinks), _stream()), "attention_heads")
 
 
 FUSED_DECODE_MAX_GROUP = 14   # query heads per kv head the fused decode kernel takes (two waves make the key and value)

@@ -1,3 +1,3 @@
 """Architectures.  Importing this package registers each of them."""
 
-from tokamak_amd.models import gubanex, qwen3, rorosun, supinex  # noqa: F401
+from tokamak_amd.models import gubanex, mepupel, qwen3, rorosun, supinex  # noqa: F401

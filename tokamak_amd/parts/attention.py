@@ -129,7 +129,8 @@ class RotatedUnitAttention(Mixer):
     q, k <- x / sqrt(mean(x^2) + ``norm_eps``) per head (``norm_eps`` None: no norm);
     score = q . k * ``softmax_scale``; with ``chunk`` = C position i sees j <= i only if
     i // C == j // C, chunks counted from position 0 of the sequence whatever the step's cut; with
-    ``window`` = W only if i - j < W; softmax; o projection over the concatenated heads.  Keys are
+    ``window`` = W only if i - j < W, or, with ``keep_first`` = F, if j < F (the first F positions of a
+    sequence stay visible at their true positions); softmax; o projection over the concatenated heads.  Keys are
     cached after rotation and norm, values as projected.  Tensors: q, k, v, o behind the part's prefix.
 
     ``sink``: every head has a learned number s_a (tensor ``sink`` [heads], float32) whose exp(s_a)
@@ -149,7 +150,7 @@ class RotatedUnitAttention(Mixer):
                  softmax_scale: float, norm_eps: float | None, chunk: int | None, dtype, device,
                  names: tuple[str, str, str, str] = ("q", "k", "v", "o"), window: int | None = None,
                  sink: bool = False, value_mix: str | None = None,
-                 extra_names: tuple[str, str] = ("sink", "vmix")) -> None:
+                 extra_names: tuple[str, str] = ("sink", "vmix"), keep_first: int = 0) -> None:
         super().__init__(dtype=dtype, device=device)
         if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})")
@@ -170,6 +171,9 @@ class RotatedUnitAttention(Mixer):
         if value_mix not in (None, "source", "mix"):
             raise ValueError(f"value_mix is None, 'source' or 'mix', got {value_mix!r}")
         self.window = None if window is None else int(window)
+        if keep_first < 0 or (keep_first and window is None):
+            raise ValueError("keep_first must be >= 0 and goes with a window")
+        self.keep_first = int(keep_first)
         self.has_sink, self.value_mix = bool(sink), value_mix
         self.extra_names = tuple(extra_names)
         self.sink: torch.Tensor | None = None
@@ -204,7 +208,8 @@ class RotatedUnitAttention(Mixer):
             self.o = wide.view(self.hidden_size, self.num_heads * self.value_size).contiguous()
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest.of(window=self.window, k=self.num_kv_heads * self.key_size, v=self.num_kv_heads * self.value_size)
+        return CacheRequest.of(window=self.window, keep_first=self.keep_first, k=self.num_kv_heads * self.key_size,
+                               v=self.num_kv_heads * self.value_size)
 
     def step_planner(self):
         return ATTENTION_WORK
@@ -217,7 +222,8 @@ class RotatedUnitAttention(Mixer):
 
     def visible_keys(self, position: int) -> int:
         if self.window is not None:
-            return min(position + 1, self.window)
+            behind = max(0, position + 1 - self.window)      # positions behind the window, of which the first stay
+            return min(position + 1, self.window) + min(behind, self.keep_first)
         return position + 1 if self.chunk is None else position % self.chunk + 1
 
     def _shared_values(self, batch, n: int, device):
@@ -257,7 +263,8 @@ class RotatedUnitAttention(Mixer):
         attended = torch.empty((n, nh * self.value_size), dtype=h.dtype, device=h.device)
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended, num_heads=nh,
                         num_kv_heads=nkv, head_dim=self.key_size, value_dim=self.value_size, page_size=store.page_size,
-                        scale=self.softmax_scale, chunk=self.chunk, window=self.window, sinks=self.sink)
+                        scale=self.softmax_scale, chunk=self.chunk, window=self.window, sinks=self.sink,
+                        keep_first=self.keep_first)
         return linear(attended, self.o, allow_partials=True)
 
 

@@ -110,15 +110,17 @@ class CacheRequest:
     width and dtype (keys and values of unlike sizes, a compressed latent beside
     its rotary part).  The mixer reads ``store.arrays[name]``, laid out
     [num_pages, elems_per_token * page_size].  ``window``: None to keep every
-    token, W if only the last W positions are ever read."""
+    token, W if only the last W positions are ever read.  ``keep_first``: with a window, the first
+    so many positions of a sequence are read for as long as it lives, and their pages stay."""
 
     arrays: tuple[tuple[str, PagedArray], ...]
     window: int | None = None
+    keep_first: int = 0
 
     @classmethod
-    def of(cls, window: int | None = None, **arrays: int | PagedArray) -> CacheRequest:
+    def of(cls, window: int | None = None, keep_first: int = 0, **arrays: int | PagedArray) -> CacheRequest:
         return cls(tuple((n, a if isinstance(a, PagedArray) else PagedArray(int(a))) for n, a in arrays.items()),
-                   window)
+                   window, int(keep_first) if window is not None else 0)
 
     def bytes_per_token(self, default_dtype: torch.dtype) -> int:
         return sum(a.elems_per_token * torch.empty((), dtype=a.dtype or default_dtype).element_size()
@@ -153,13 +155,17 @@ class PositionData:
 
 @dataclass
 class BranchPair:
-    """The outputs of two sub-layers that read the same normed input, not yet added to the residual
-    stream: each [N, H] in the compute dtype or float32, or float32 partial sums [P, N, H];
-    ``second`` may be None.  The norm that reads the stream next forms first + second in float32 and
-    adds the sum to the stream once."""
+    """The outputs of up to three sub-layers (or terms of one) that belong to one residual add, not
+    yet added to the stream: each [N, H] in the compute dtype or float32, or float32 partial sums
+    [P, N, H]; ``second`` and ``third`` may be None.  ``bias``: None or float32 [H], one more term,
+    the same for every row.  The norm that reads the stream next forms
+    scale * (first + second + third + bias) in float32 and adds it to the stream once."""
 
     first: torch.Tensor
     second: torch.Tensor | None = None
+    third: torch.Tensor | None = None
+    bias: torch.Tensor | None = None
+    scale: float = 1.0
 
 
 class Embedding(Part):
@@ -217,7 +223,10 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
+    """``forward`` returns the sub-layer's output, or a tuple of up to two terms whose sum it is (a
+    mixture's routed experts and its shared expert): whoever adds the output to the stream adds the terms."""
+
+    def forward(self, h: torch.Tensor, batch) -> "torch.Tensor | tuple[torch.Tensor, ...]":
         raise NotImplementedError
 
 

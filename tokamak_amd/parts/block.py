@@ -46,7 +46,12 @@ class PreNormBlock(Block):
         pending = self.mixer.forward(h, batch, store, writes_cache, position, **into)
         h = _normed(self.feed_forward_norm, resid, pending, self.feed_forward)
         into = _sink(self.feed_forward, then, resid)
-        return self.feed_forward.forward(h, batch, **into)
+        return _whole(self.feed_forward.forward(h, batch, **into))
+
+
+def _whole(out):
+    """A feed-forward's output as one pending sub-layer output (its terms, if it has several, as a pair)."""
+    return BranchPair(*out) if isinstance(out, tuple) else out
 
 
 def _normed(norm, resid, pending, consumer):
@@ -111,32 +116,57 @@ class ParallelMixersBlock(Block):
 
 
 class ParallelSublayersBlock(Block):
-    """h = norm(x); x = x + (mixer(h) + feed_forward(h)).
+    """h = norm(x); x = x + branch_scale * (mixer(h) + feed_forward(h)).
 
-    One norm; the mixer and the feed-forward both read its output, and their outputs are added to
-    each other first and to the residual stream once, in float32, by the norm that reads the stream
-    next (it receives them as a ``BranchPair``).  The feed-forward may be absent: x = x + mixer(h).
+    The mixer and the feed-forward read the same stream, and their outputs are added to each other
+    first and to the residual stream once, in float32, by the norm that reads the stream next (it
+    receives them as a ``BranchPair``).  With a ``feed_forward_norm`` the feed-forward has a norm of
+    its own over the same x: x = x + branch_scale * (mixer(norm(x)) + feed_forward(feed_forward_norm(x)));
+    where the two norms agree on everything but their weights one kernel makes both outputs.  The
+    feed-forward may be absent: x = x + branch_scale * mixer(h).  A feed-forward may return two terms
+    (routed and shared experts) and leave a bias of its last product to the add (``output_bias``).
     An optional ``position`` part prepares the step's position data for the mixer.
     """
 
     roles = ("norm", "mixer")
-    optional = ("position", "feed_forward")
+    optional = ("position", "feed_forward", "feed_forward_norm")
     replays_parts = True
 
-    def __init__(self, parts) -> None:
+    def __init__(self, parts, *, branch_scale: float = 1.0) -> None:
         super().__init__(parts)
+        self.branch_scale = float(branch_scale)
         self.norm = parts["norm"]
         self.feed_forward = parts.get("feed_forward")
+        self.feed_forward_norm = parts.get("feed_forward_norm")
+        if self.feed_forward_norm is not None and self.feed_forward is None:
+            raise ValueError("a feed-forward norm without a feed-forward")
         self.position = parts.get("position")
         self.entry_norm = self.norm
 
+    def _normed(self, resid, pending):
+        """(the mixer's input, the feed-forward's)."""
+        if self.feed_forward_norm is None:
+            h = self.norm.forward(resid, pending)
+            return h, h
+        pair = getattr(self.norm, "forward_pair", None)
+        both = pair(self.feed_forward_norm, resid, pending) if pair is not None else None
+        if both is not None:
+            return both
+        h = self.norm.forward(resid, pending)
+        return h, self.feed_forward_norm.forward(resid, None)
+
     def forward(self, resid, pending, batch, store, writes_cache):
         position = None if self.position is None else self.position.prepare(batch)
-        h = self.norm.forward(resid, pending)
+        h, h_ff = self._normed(resid, pending)
         mixed = self.mixer.forward(h, batch, store, writes_cache, position)
         if self.feed_forward is None:
-            return mixed
-        return BranchPair(mixed, self.feed_forward.forward(h, batch))
+            return mixed if self.branch_scale == 1.0 else BranchPair(mixed, scale=self.branch_scale)
+        bias = getattr(self.feed_forward, "output_bias", None)
+        out = self.feed_forward.forward(h_ff, batch, defer_bias=True) if bias is not None else self.feed_forward.forward(h_ff, batch)
+        terms = out if isinstance(out, tuple) else (out,)
+        if len(terms) > 2:
+            raise ValueError("a feed-forward hands on two terms at most")
+        return BranchPair(mixed, *terms, bias=bias, scale=self.branch_scale)
 
 
 register_part("block", "pre_norm", PreNormBlock)

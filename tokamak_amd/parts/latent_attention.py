@@ -30,6 +30,12 @@ class LatentAttention(Mixer):
     latents with ``num_heads`` query heads on one kv head, and the head's result, a weighted sum of
     latents, goes through W_uv,a afterwards; the up-projections of cached tokens are never formed.
     Tensors: q, dkv, dkv.norm, uk, uv, o (and sink) behind the part's prefix.
+
+    ``q_rank``: the queries go through a latent of their own, c_q = W_dq h divided by its root mean
+    square (``norm_eps``) times a weight, q = W_uq c_q (tensors dq, dq.norm, uq in place of q; without
+    a rotated part).
+    ``own_latent`` False: the layer has no W_dkv and caches nothing; it attends over the latents that
+    another layer of the same rank left in the cache slot its call names, with its own W_uk and W_uv.
     """
 
     capturable = True
@@ -37,7 +43,9 @@ class LatentAttention(Mixer):
 
     def __init__(self, *, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, rank: int,
                  softmax_scale: float, norm_eps: float, window: int | None, sink: bool, dtype, device,
-                 names: tuple[str, ...] = ("q", "dkv", "dkv.norm", "uk", "uv", "o", "sink")) -> None:
+                 names: tuple[str, ...] = ("q", "dkv", "dkv.norm", "uk", "uv", "o", "sink"),
+                 q_rank: int | None = None, own_latent: bool = True,
+                 q_names: tuple[str, str, str] = ("dq", "dq.norm", "uq")) -> None:
         super().__init__(dtype=dtype, device=device)
         if min(hidden_size, num_heads, head_dim, value_dim, rank) < 1 or rot_dim < 0:
             raise ValueError("every size of the latent attention must be >= 1 (rot_dim >= 0)")
@@ -54,14 +62,28 @@ class LatentAttention(Mixer):
         self.window = None if window is None else int(window)
         self.has_sink = bool(sink)
         self.names = tuple(names)
+        self.q_rank = None if q_rank is None else int(q_rank)
+        if self.q_rank is not None and not 1 <= self.q_rank <= 1024:
+            raise ValueError(f"q_rank must be 1 to 1,024, got {q_rank}")
+        if self.q_rank is not None and self.rot_dim:
+            raise ValueError("queries through a latent have no rotated part here (rot_dim must be 0)")
+        self.own_latent = bool(own_latent)
+        self.q_names = tuple(q_names)
         self.q_dkv = self.latent_norm = self.uk_t = self.uv = self.o = self.sink = None
+        self.q_norm = self.uq = None
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         h, nh, hd, rd, vd, r = self.hidden_size, self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank
         q, dkv, norm, uk, uv, o, sink = self.names
-        out = {prefix + q: TensorSpec((nh * (hd + rd), h)), prefix + dkv: TensorSpec((r + rd, h)),
-               prefix + norm: TensorSpec((r,), role="vector"), prefix + uk: TensorSpec((nh * hd, r)),
-               prefix + uv: TensorSpec((nh * vd, r)), prefix + o: TensorSpec((h, nh * vd))}
+        out = {prefix + uk: TensorSpec((nh * hd, r)), prefix + uv: TensorSpec((nh * vd, r)), prefix + o: TensorSpec((h, nh * vd))}
+        if self.own_latent:
+            out.update({prefix + dkv: TensorSpec((r + rd, h)), prefix + norm: TensorSpec((r,), role="vector")})
+        if self.q_rank is None:
+            out[prefix + q] = TensorSpec((nh * (hd + rd), h))
+        else:
+            dq, dq_norm, uq = self.q_names
+            out.update({prefix + dq: TensorSpec((self.q_rank, h)), prefix + dq_norm: TensorSpec((self.q_rank,), role="vector"),
+                        prefix + uq: TensorSpec((nh * (hd + rd), self.q_rank))})
         if self.has_sink:
             out[prefix + sink] = TensorSpec((nh,), role="vector")
         return out
@@ -69,9 +91,13 @@ class LatentAttention(Mixer):
     def bind(self, prefix: str, fetch: Fetch) -> None:
         q, dkv, norm, uk, uv, o, sink = self.names
         nh, hd, vd, r = self.num_heads, self.head_dim, self.value_dim, self.rank
-        # one product yields the queries, the latent and the rotated key part
-        self.q_dkv = torch.cat([fetch(prefix + q), fetch(prefix + dkv)], dim=0).contiguous()
-        self.latent_norm = fetch(prefix + norm)
+        # one product yields the queries (or their latent), the latent and the rotated key part
+        first = fetch(prefix + q) if self.q_rank is None else fetch(prefix + self.q_names[0])
+        self.q_dkv = torch.cat([first, fetch(prefix + dkv)], dim=0).contiguous() if self.own_latent else first
+        self.latent_norm = fetch(prefix + norm) if self.own_latent else None
+        if self.q_rank is not None:
+            self.q_norm = fetch(prefix + self.q_names[1])
+            self.uq = fetch(prefix + self.q_names[2])
         # W_uk per head, transposed: [heads, rank, head_dim] takes a query into the latent's space
         self.uk_t = fetch(prefix + uk).view(nh, hd, r).transpose(1, 2).contiguous()
         self.uv = fetch(prefix + uv).view(nh, vd, r).contiguous()
@@ -79,7 +105,9 @@ class LatentAttention(Mixer):
         if self.has_sink:
             self.sink = fetch(prefix + sink)
 
-    def cache_request(self) -> CacheRequest:
+    def cache_request(self) -> CacheRequest | None:
+        if not self.own_latent:
+            return None
         return CacheRequest.of(window=self.window, k=self.key_size, v=self.value_size)
 
     def step_planner(self):
@@ -97,7 +125,10 @@ class LatentAttention(Mixer):
     def forward(self, h, batch, store, writes_cache: bool = True, position: PositionData | None = None):
         nh, hd, rd, vd, r = self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank
         n = h.shape[0]
-        weight = self.q_dkv if writes_cache else self.q_dkv[: nh * (hd + rd)]
+        if writes_cache and not self.own_latent:
+            raise ops.KernelError("a latent attention without a latent of its own reads another layer's cache slot")
+        q_rows = nh * (hd + rd) if self.q_rank is None else self.q_rank
+        weight = self.q_dkv if writes_cache or not self.own_latent else self.q_dkv[:q_rows]
         proj = linear(h, weight, allow_partials=True)
         cos = sin = None
         rotary_dim, interleaved = 0, False
@@ -106,12 +137,28 @@ class LatentAttention(Mixer):
                 raise ops.KernelError("this attention part has no kernel for a bias on the scores")
             cos, sin, rotary_dim, interleaved = position.cos, position.sin, position.rotary_dim, position.interleaved
         tables = batch.block_tables[store.group]
-        q_plain = torch.empty((n, nh, hd), dtype=h.dtype, device=h.device)
         q_full = torch.empty((n, nh, self.key_size), dtype=h.dtype, device=h.device)
-        ops.latent_prepare(proj, self.latent_norm, cos, sin, batch.positions, batch.req_of_token, tables, q_plain, q_full,
-                           store.arrays["k"], store.arrays["v"], num_heads=nh, head_dim=hd, rot_dim=rd, rank=r,
-                           rotary_dim=rotary_dim, interleaved=interleaved, page_size=store.page_size, eps=self.norm_eps,
-                           store=writes_cache)
+        if self.q_rank is None:
+            q_plain = torch.empty((n, nh, hd), dtype=h.dtype, device=h.device)
+            ops.latent_prepare(proj, self.latent_norm, cos, sin, batch.positions, batch.req_of_token, tables, q_plain, q_full,
+                               store.arrays["k"], store.arrays["v"], num_heads=nh, head_dim=hd, rot_dim=rd, rank=r,
+                               rotary_dim=rotary_dim, interleaved=interleaved, page_size=store.page_size, eps=self.norm_eps,
+                               store=writes_cache)
+        else:
+            # the query's latent is one unit that is normed like the keys' latent, which goes into the pages
+            c_q = torch.empty((n, self.q_rank), dtype=h.dtype, device=h.device)
+            ops.latent_prepare(proj, self.latent_norm, None, None, batch.positions, batch.req_of_token, tables, c_q, None,
+                               store.arrays["k"], store.arrays["v"], num_heads=1, head_dim=self.q_rank, rot_dim=0, rank=r,
+                               rotary_dim=0, interleaved=False, page_size=store.page_size, eps=self.norm_eps,
+                               store=writes_cache, q_weight=self.q_norm)
+            q = linear(c_q, self.uq)
+            if self.key_size == r:
+                q_plain = q.view(n, nh, hd)
+            else:
+                q_plain = torch.empty((n, nh, hd), dtype=h.dtype, device=h.device)
+                ops.latent_prepare(q, None, cos, sin, batch.positions, batch.req_of_token, tables, q_plain, q_full,
+                                   None, None, num_heads=nh, head_dim=hd, rot_dim=rd, rank=r, rotary_dim=rotary_dim,
+                                   interleaved=interleaved, page_size=store.page_size, eps=self.norm_eps, store=False)
         ops.head_linear(q_plain, self.uk_t, q_full[:, :, :r])
         attended = torch.empty((n, nh, self.value_size), dtype=h.dtype, device=h.device)
         paged_attention(q_full, store.arrays["k"], store.arrays["v"], tables, batch, attended, num_heads=nh,

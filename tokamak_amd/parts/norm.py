@@ -54,12 +54,28 @@ class RMSNorm(Norm):
         m = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((m, self.dim), dtype=self.dtype, device=resid.device)
         if isinstance(delta, BranchPair):
-            # two branches that read the same normed input: their sum is formed first, then added
+            # branches that belong to one residual add: their sum is formed first, then added
             ops.add_norm2(resid, delta.first, delta.second, self.weight, self.eps, out, center=False, rows=rows,
-                          write_resid=write_resid)
+                          write_resid=write_resid, c=delta.third, bias=delta.bias, scale=delta.scale)
             return out
         ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows=rows, write_resid=write_resid)
         return out
+
+    def forward_pair(self, other: "RMSNorm", resid, delta):
+        """(this norm's output, ``other``'s) of the same stream resid + delta, from one kernel: the row's root
+        mean square is formed once and the row leaves twice, each time with one of the two weights.  None if
+        the two norms do not agree on the size and eps (the caller then runs them one after the other)."""
+        if type(other) is not type(self) or other.dim != self.dim or other.eps != self.eps or other.dtype != self.dtype:
+            return None
+        if isinstance(delta, Added):
+            delta = None
+        pair = delta if isinstance(delta, BranchPair) else BranchPair(delta) if delta is not None else None
+        out = torch.empty((resid.shape[0], self.dim), dtype=self.dtype, device=resid.device)
+        out2 = torch.empty_like(out)
+        ops.add_norm2(resid, pair.first if pair else None, pair.second if pair else None, self.weight, self.eps, out,
+                      center=False, c=pair.third if pair else None, bias=pair.bias if pair else None,
+                      scale=pair.scale if pair else 1.0, weight2=other.weight, out2=out2)
+        return out, out2
 
 
 class ScalarRMSNorm(RMSNorm):
@@ -98,10 +114,11 @@ class LayerNorm(Norm):
         self.weight = fetch(prefix + self.tensor)
 
     def forward(self, resid, delta, *, rows=None, write_resid=True):
-        first, second = (delta.first, delta.second) if isinstance(delta, BranchPair) else (delta, None)
+        pair = delta if isinstance(delta, BranchPair) else BranchPair(delta)
         m = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((m, self.dim), dtype=self.dtype, device=resid.device)
-        ops.add_norm2(resid, first, second, self.weight, self.eps, out, center=True, rows=rows, write_resid=write_resid)
+        ops.add_norm2(resid, pair.first, pair.second, self.weight, self.eps, out, center=True, rows=rows,
+                      write_resid=write_resid, c=pair.third, bias=pair.bias, scale=pair.scale)
         return out
 
 

@@ -23,24 +23,35 @@ class RotaryHalf(PositionEncoding):
     l = 2 pi / f: kept where l < original / high, divided by ``factor`` where l > original / low,
     and in between (1 - s) f / factor + s f with s = (original / l - low) / (high - low);
     computed on the host in double precision, then rounded to float32 once.
+
+    ``yarn`` = (factor, original, fast, slow) stretches the slow frequencies with a ramp over the
+    dimensions instead and multiplies both tables by 0.1 ln(factor) + 1 (``yarn_frequencies``).
     """
 
     capturable = True
     replayable = True
 
-    def __init__(self, *, rotary_dim: int, theta: float, dtype, device, scaling: tuple | None = None) -> None:
+    def __init__(self, *, rotary_dim: int, theta: float, dtype, device, scaling: tuple | None = None,
+                 yarn: tuple | None = None) -> None:
         super().__init__(dtype=dtype, device=device)
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
+        if scaling is not None and yarn is not None:
+            raise ValueError("frequencies are rescaled by wavelength or stretched by a ramp, not both")
         self.rotary_dim = int(rotary_dim)
         self.theta = float(theta)
         self.scaling = None if scaling is None else tuple(float(x) for x in scaling)
-        if self.scaling is None:
+        self.yarn = None if yarn is None else tuple(float(x) for x in yarn)
+        self.amplitude = 1.0
+        if self.yarn is not None:
+            freqs, self.amplitude = yarn_frequencies(self.rotary_dim, self.theta, self.yarn)
+            inv_freq = torch.tensor(freqs, dtype=torch.float64).to(torch.float32)
+        elif self.scaling is None:
             inv_freq = 1.0 / (self.theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
         else:
             inv_freq = torch.tensor(scaled_frequencies(self.rotary_dim, self.theta, *self.scaling), dtype=torch.float32)
         self.inv_freq = inv_freq.to(self.device)
-        self.key = ("rotary_half", self.rotary_dim, self.theta, self.scaling)
+        self.key = ("rotary_half", self.rotary_dim, self.theta, self.scaling, self.yarn)
 
     def prepare(self, batch) -> PositionData:
         """cos and sin, each float32 [N, rotary_dim/2]; computed once per step."""
@@ -49,7 +60,7 @@ class RotaryHalf(PositionEncoding):
             n, half = batch.num_tokens, self.rotary_dim // 2
             cos = torch.empty((n, half), dtype=torch.float32, device=self.device)
             sin = torch.empty((n, half), dtype=torch.float32, device=self.device)
-            ops.rope_tables(batch.positions, self.inv_freq, cos, sin)
+            ops.rope_tables(batch.positions, self.inv_freq, cos, sin, self.amplitude)
             cached = batch.memo[self.key] = PositionData(cos=cos, sin=sin, rotary_dim=self.rotary_dim)
         return cached
 
