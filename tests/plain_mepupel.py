@@ -166,9 +166,11 @@ def gated(h: torch.Tensor, w: dict, p: str, biases: bool) -> torch.Tensor:
     return out + _f(w[p + "down.b"]) if biases else out
 
 
-def route(h: torch.Tensor, w: dict, p: str, router: dict) -> tuple[torch.Tensor, torch.Tensor]:
-    """(chosen experts [T, top], their weights [T, top])."""
+def route(h: torch.Tensor, w: dict, p: str, router: dict, margins: list | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """(chosen experts [T, top], their weights [T, top]).  ``margins`` receives, per token, the narrowest
+    gap of a choice score (of a group or of an expert) between what was taken and what was not."""
     experts, top = int(router["experts"]), int(router["top"])
+    gap = torch.full((h.shape[0],), float("inf"), dtype=DTYPE)
     s = torch.sigmoid(h @ _f(w[p + "router"]).T)
     choice = s + _f(w[p + "correction"])[None, :] if p + "correction" in w else s.clone()
     groups = router.get("groups")
@@ -177,17 +179,25 @@ def route(h: torch.Tensor, w: dict, p: str, router: dict) -> tuple[torch.Tensor,
         size = experts // count
         grouped = choice.view(-1, count, size)
         score = grouped.topk(min(2, size), dim=-1).values.sum(dim=-1)          # [T, count]
+        if keep < count:
+            ordered = score.sort(dim=-1, descending=True).values
+            gap = torch.minimum(gap, ordered[:, keep - 1] - ordered[:, keep])
         kept = torch.zeros_like(score, dtype=torch.bool)
         kept.scatter_(1, score.topk(keep, dim=-1).indices, True)
         choice = choice.masked_fill(~kept[:, :, None].expand(-1, -1, size).reshape(-1, experts), float("-inf"))
     chosen = choice.topk(top, dim=-1).indices
+    if top < experts:
+        ordered = choice.sort(dim=-1, descending=True).values
+        gap = torch.minimum(gap, ordered[:, top - 1] - ordered[:, top])     # (inf where nothing else may be chosen)
+    if margins is not None:
+        margins.extend(gap.tolist())
     weight = s.gather(1, chosen)
     weight = weight / (weight.sum(dim=-1, keepdim=True) + 1e-20) * float(router.get("scale", 1.0))
     return chosen, weight
 
 
-def experts_ff(h: torch.Tensor, w: dict, p: str, mlp: dict) -> torch.Tensor:
-    chosen, weight = route(h, w, p, mlp["router"])
+def experts_ff(h: torch.Tensor, w: dict, p: str, mlp: dict, margins: list | None = None) -> torch.Tensor:
+    chosen, weight = route(h, w, p, mlp["router"], margins)
     out = torch.zeros_like(h)
     for i in range(h.shape[0]):
         for e, x in zip(chosen[i].tolist(), weight[i]):
@@ -197,17 +207,18 @@ def experts_ff(h: torch.Tensor, w: dict, p: str, mlp: dict) -> torch.Tensor:
     return out
 
 
-def feed_forward(h: torch.Tensor, w: dict, p: str, mlp: dict | None) -> torch.Tensor | None:
+def feed_forward(h: torch.Tensor, w: dict, p: str, mlp: dict | None, margins: list | None = None) -> torch.Tensor | None:
     if mlp is None:
         return None
     if mlp["kind"] == "dense":
         return gated(h, w, p, True)
-    return experts_ff(h, w, p, mlp)
+    return experts_ff(h, w, p, mlp, margins)
 
 
 # ---------------------------------------------------------------------------------------------
-def forward(cfg: dict, w: dict, tokens: list[int]) -> tuple[torch.Tensor, torch.Tensor]:
-    """(logits [T, vocab], the residual stream after every layer [layers, T, width])."""
+def forward(cfg: dict, w: dict, tokens: list[int], margins: list | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """(logits [T, vocab], the residual stream after every layer [layers, T, width]).  ``margins`` receives the
+    routers' narrowest choices, T numbers for every layer with a mixture of experts, in layer order."""
     eps = float(cfg["norm"]["eps"])
     mult = float(cfg.get("residual_mult", 1.0))
     x = _f(w["embed"])[torch.tensor(tokens, dtype=torch.long)]
@@ -230,7 +241,7 @@ def forward(cfg: dict, w: dict, tokens: list[int]) -> tuple[torch.Tensor, torch.
         else:
             raise ValueError(layer["type"])
         if layer.get("mlp") is not None:
-            mixed = mixed + feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"])
+            mixed = mixed + feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"], margins)
         x = x + mult * mixed
         after.append(x)
     logits = rms_norm(x, w["final.norm"], eps) @ _f(w["head"]).T

@@ -114,7 +114,7 @@ class GroupTables:
         if table is None:
             return 0
         lo = self.first_live.get(request, self.kept_pages)
-        hi = min(max(first_needed_position // self.page_size, lo), len(table))
+        hi = max(lo, min(first_needed_position // self.page_size, len(table)))
         self.pool.give_back(table[i] for i in range(lo, hi))
         for i in range(lo, hi):
             table[i] = RELEASED
@@ -128,7 +128,7 @@ class GroupTables:
         if table is None:
             return 0
         lo = self.first_live.get(request, self.kept_pages)
-        return max(0, min(max(first_needed_position // self.page_size, lo), len(table)) - lo)
+        return max(lo, min(first_needed_position // self.page_size, len(table))) - lo
 
     def free(self, request) -> None:
         table = self.tables.pop(request, None)

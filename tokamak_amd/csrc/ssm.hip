@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
   const int first = q_start[req], end = q_start[req + 1];
   const int t_lo = first + blockIdx.z * kConvSegment, t_hi = min(end, t_lo + kConvSegment);
   if (c >= C || t_lo >= end) return;
-  float* st = state + (size_t)state_slots[req] * (taps - 1) * C + c;
+  float* st = taps > 1 ? state + (size_t)state_slots[req] * (taps - 1) * C + c : nullptr;
   // taps and window sit at the END of arrays of kMaxTaps: index kMaxTaps - 1 is the token itself
   float wv[kMaxTaps], win[kMaxTaps];
 #pragma unroll
