@@ -390,7 +390,7 @@ def test_grouped_router_and_experts_with_a_shared_one(dtype, name, correction):
         margins: list = []
         chosen, weight = plain.route(h.double(), double(w), "l0.mlp.", mlp["router"], margins)
         clear = torch.tensor(margins) > (NARROW if dtype == torch.bfloat16 else 1e-5)
-        assert rows < 100 or int(clear.sum()) >= rows // 3
+        assert rows < 100 or int(clear.sum()) >= rows // 5
         if not bool(clear.any()):
             continue
         got_chosen = torch.empty((rows, r["top"]), dtype=torch.int32, device=DEV)
