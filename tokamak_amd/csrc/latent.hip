@@ -49,10 +49,19 @@ __global__ void latent_prepare_kernel(
   const int plain = is_q ? dim : rank;      // elements before the rotated part
   const TIN* src = proj + (size_t)n * row_width + (is_q ? (size_t)a * qw : (size_t)nh * qw);
   float* vec = vecs[wave];
-  for (int d = lane; d < width; d += kWave) {
-    float v = 0.f;
-    for (int p = 0; p < parts; ++p) v += Elem<TIN>::load(src + (size_t)p * part_stride + d);
-    vec[d] = v;
+  // four elements a lane at a time, each summed over the parts in order: their loads are all in flight
+  for (int d0 = lane; d0 < width; d0 += 4 * kWave) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < parts; ++p) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int d = min(d0 + u * kWave, width - 1);      // (past the end: the last element again, not kept)
+        v[u] += Elem<TIN>::load(src + (size_t)p * part_stride + d);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (d0 + u * kWave < width) vec[d0 + u * kWave] = v[u];
   }
   wave_lds_sync();
   // rotation of the first `rot` dims of the rotated part

@@ -27,8 +27,10 @@ WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles 
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
 GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays
 GROUP_FILL = 128                # ... if its blocks times their shares of the keys are at least this many (half the CUs)
-HEADS_FORM_FROM_GROUP = 8       # query heads a kv head from which tokens that run alone take ops.attention_heads (the
-                                # heads are a product's 16 columns: with fewer, most of a product is idle)
+HEADS_FORM_FROM_GROUP = 4       # query heads a kv head from which tokens that run alone take ops.attention_heads (the
+                                # heads are a product's 16 columns: with fewer, most of a product is idle; with four a
+                                # token over a window of 1,024 keys of 128 channels still takes 22 us against 44 in
+                                # the generic kernel)
 TILES_ON_MATRIX_CORES = True    # bfloat16 portions that the tuned kernels do not take: csrc/attention_tiles.hip rather than
                                 # the generic kernel (tests of the generic kernel's own tiles switch this off)
 

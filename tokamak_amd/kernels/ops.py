@@ -281,7 +281,8 @@ _SIGS = {
         "tk_conv_silu": [c_int, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_ssd_scan": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p, c_void_p,
-                        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                        c_void_p, c_void_p, c_void_p],
         "tk_gated_group_norm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_void_p, c_void_p,
                                 c_int, c_int, c_int, c_float, c_void_p],
     },
@@ -935,6 +936,8 @@ SSM_MAX_TAPS = 8             # taps of the short convolution (csrc/ssm.hip: kMax
 SSM_SPLIT_FROM_TOKENS = 64   # a request's tokens in a step from which a head's value columns are shared out
 SSM_SPLIT_MIN_COLUMNS = 8
 SSM_SPLIT_BLOCKS = 1024
+SSM_CHUNK_TOKENS = 64        # tokens of a chunk of a long portion; the chunks of a portion run side by side
+SSM_CHUNKS_FROM_TOKENS = 128  # a request's tokens in a step from which the step's portions are cut into chunks
 
 
 def _ssm_in(t: torch.Tensor, rows: int, dtype: torch.dtype, what: str):
@@ -999,11 +1002,24 @@ def ssd_scan(u: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Te
     _need(1 <= vdim <= 1024 and 1 <= state_size <= 1024 and batch.num_tokens == n, "the scan takes sizes up to 1,024")
     pointer, is_f32, parts, stride, ld = _ssm_in(proj, n, u.dtype, "projections")
     _need(0 <= dt_col and dt_col + heads <= ld, "the step sizes lie outside the projections")
-    splits = ssd_column_splits(batch.num_requests, heads, vdim, batch.max_q_len)
+    # Long portions: chunks of SSM_CHUNK_TOKENS tokens side by side (a chunk acts on the state as S -> P S + L, with P
+    # and L found from zeros; the chunks' start states follow from those in order; then every chunk runs again
+    # from its own start and writes its outputs): twice the arithmetic of one walk, a thirtieth of its length.
+    chunk = max_chunks = 0
+    chunk_state = chunk_decay = None
+    blocks = batch.num_requests
+    if batch.max_q_len >= SSM_CHUNKS_FROM_TOKENS:
+        chunk = SSM_CHUNK_TOKENS
+        max_chunks = -(-batch.max_q_len // chunk)
+        blocks = n // chunk + batch.num_requests        # (no step has more chunks than this)
+        chunk_state = torch.empty((blocks, heads, state_size, vdim), dtype=torch.float32, device=y.device)
+        chunk_decay = torch.empty((blocks, heads), dtype=torch.float32, device=y.device)
+    splits = ssd_column_splits(blocks, heads, vdim, batch.max_q_len)
     _note(f"{n}x{heads}x{state_size}x{vdim}", n * (c * u.element_size() + heads * vdim * 4), 6.0 * n * heads * state_size * vdim)
     _check(_fn("ssm", "tk_ssd_scan")(_code(u.dtype), _p(u), pointer, is_f32, parts, stride, ld, int(dt_col), _p(dt_bias),
                                      _p(a_log), _p(skip), _p(state), _p(batch.q_start), _p(batch.state_slots), _p(y),
-                                     batch.num_requests, heads, groups, state_size, vdim, splits, _stream()), "ssd_scan")
+                                     batch.num_requests, heads, groups, state_size, vdim, splits, chunk, max_chunks,
+                                     _p(chunk_state), _p(chunk_decay), _stream()), "ssd_scan")
 
 
 def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, weight: torch.Tensor, out: torch.Tensor, *,
