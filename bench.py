@@ -746,7 +746,8 @@ def main() -> int:
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
     ap.add_argument("--pairs", default="rorosun-0.6b:qwen3-0.6b,rorosun-8b:qwen3-8b",
                     help="compare workload: NEW:OLD preset pairs, each measured like --shape "
-                         "(for instance gubanex-0.6b:qwen3-0.6b,gubanex-8b:qwen3-8b or supinex-0.6b:gubanex-0.6b,supinex-8b:gubanex-8b)")
+                         "(for instance gubanex-0.6b:qwen3-0.6b,gubanex-8b:qwen3-8b, supinex-0.6b:gubanex-0.6b,supinex-8b:gubanex-8b "
+                         "or mepupel-0.6b:supinex-0.6b,mepupel-8b:supinex-8b with --layers 6)")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--max-batch", type=int, default=64)
     ap.add_argument("--prompt-tokens", default="32,1024", help="continuous workload: MIN,MAX prompt length")
