@@ -200,7 +200,10 @@ def test_state_space_mixer_in_portions_over_state_slots(dtype, name):
         step += 1
     for r in lengths:
         close(torch.cat(got[r]), want[r][0].float(), dtype, slack=2.0)
-        close(store.state["S"][slots[r]].cpu(), want[r][1].float(), dtype, slack=2.0)
+        held = store.state["S"][slots[r]].cpu()          # [heads, groups of four columns, state, 4]
+        state = held.permute(0, 2, 1, 3).reshape(m["heads"], m["state"], -1)
+        close(state[:, :, :m["vdim"]], want[r][1].float(), dtype, slack=2.0)
+        assert bool((state[:, :, m["vdim"]:] == 0).all())
     for array in store.state.values():
         assert bool((array[3] == 7.0).all()) and bool((array[1] == 0.0).all())
     if m["conv"] > 1:

@@ -126,13 +126,48 @@ __global__ __launch_bounds__(256) void conv_carry_kernel(
     if (j < taps - 1) st[(size_t)j * C] = keep[j];
 }
 
+// Sums over the KS neighbouring lanes that share a column group, for the COUNT values v[0 .. COUNT) that
+// every lane holds: at each step a lane keeps one half of its values and hands the other half to the lane
+// M away, which keeps that half (the lane whose bit M is set keeps the upper one), so that the numbers
+// that travel halve from step to step (31 exchanges for 32 values over 32 lanes, where summing every value
+// over all lanes takes 160).  Afterwards lane ks holds, in v[0 .. max(COUNT / KS, 1)), the complete sums of
+// the values from index ks * COUNT / KS on (with more lanes than values: of value ks / (KS / COUNT), in
+// every lane of that run).
+template <int COUNT, int M>
+__device__ __forceinline__ void sum_and_deal(float (&v)[32], int ks) {
+  if constexpr (M >= 1) {
+    if constexpr (COUNT > 1) {
+      constexpr int H = COUNT / 2;
+      const bool upper = (ks & M) != 0;
+#pragma unroll
+      for (int i = 0; i < H; ++i) {
+        const float send = upper ? v[i] : v[i + H];
+        const float keep = upper ? v[i + H] : v[i];
+        v[i] = keep + __shfl_xor(send, M, kWave);
+      }
+      sum_and_deal<H, M / 2>(v, ks);
+    } else {
+      v[0] += __shfl_xor(v[0], M, kWave);
+      sum_and_deal<1, M / 2>(v, ks);
+    }
+  }
+}
+
 struct ScanShape {
   int heads, groups, ns, vdim;      // ns: the state's size per value channel
-  int columns, slices, slice;       // threads = columns * slices; a thread owns `slice` state rows of a value column
+  int columns;                      // groups of four value columns that a block holds
+  int slices;                       // threads that share a column group, each with RS rows of the state (a power of two)
 };
 
 // A block a (request, head, share of the value columns).  u: the convolution's output [N, C] = [x | B | C].
 // dt_in: rows ld long, the heads' step sizes from column dt_col.  y: float32 [N, heads * vdim].
+//
+// A thread owns RS rows by four columns of the state in registers, so that the 16-byte pieces of dt B
+// and C it reads from LDS for a token serve four columns each (a thread that owns one column reads a
+// B and a C for every multiply-add pair, and the kernel is then bound by LDS reads: 1.78 -> 1.07 ms for
+// 2,048 tokens of 128 heads of 128 x 64).  The KS threads that share a column group are neighbouring
+// lanes of one wave: the outputs of a round's eight tokens are summed over them with lane exchanges
+// (sum_and_deal: no LDS array, no barrier), and every lane writes the sums it is left with.
 //
 // Long portions are cut into chunks of `chunk` tokens that run side by side (the decay is one number a
 // head and token, so a chunk's effect on the state is S_end = P S_start + L with P the product of its
@@ -142,20 +177,19 @@ struct ScanShape {
 //   MODE 2: the same blocks again, each from its S_start, with the outputs.
 // MODE 0 walks a request's tokens in one block from the request's state.  A chunk's place in the scratch
 // arrays is its number among all chunks of the step (requests in order).
-template <typename T, int SLICE, int MODE>
+template <typename T, int RS, int KS, int MODE>
 __global__ __launch_bounds__(1024) void ssd_scan_kernel(
     const T* __restrict__ u, int C, SsmIn dt_in, long ld, int dt_col, const float* __restrict__ dt_bias,
     const float* __restrict__ a_log, const float* __restrict__ skip, float* __restrict__ state,
     const int* __restrict__ q_start, const int* __restrict__ state_slots, float* __restrict__ y, ScanShape sh,
     int chunk, int max_chunks, float* __restrict__ chunk_state, float* __restrict__ chunk_decay) {
-  constexpr int TB = kScanTokens;
-  extern __shared__ float lds[];
-  const int ns = sh.ns, vdim = sh.vdim, CT = sh.columns, KS = sh.slices, slice = sh.slice;
-  const int nsp = (ns + 3) & ~3;
+  constexpr int TB = kScanTokens, CS = 4;
+  constexpr int nsp = KS * RS;       // rows with the padding (zeros behind ns)
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* bb = lds;                   // [TB][nsp]: dt B
   float* cc = bb + TB * nsp;         // [TB][nsp]: C
   float* aa = cc + TB * nsp;         // [TB]: the decay
-  float* part = aa + TB;             // [KS][TB][CT]
+  const int ns = sh.ns, vdim = sh.vdim;
   const int req = MODE == 0 ? blockIdx.x : blockIdx.x / max_chunks, head = blockIdx.y;
   int first = q_start[req];
   int end = q_start[req + 1];
@@ -170,79 +204,98 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(
     end = min(end, first + chunk);
   }
   const int tid = threadIdx.x, nthreads = blockDim.x;
-  const int ks = tid / CT, jl = tid - ks * CT;
-  const int j = blockIdx.z * CT + jl;
-  const bool worker = ks < KS;
-  const bool live = worker && j < vdim;
-  const int k0 = ks * slice;
-  const int kn = max(0, min(slice, ns - k0));
+  const int ks = tid & (KS - 1), jl = tid / KS;
+  const int j0 = (blockIdx.z * sh.columns + jl) * CS;       // the thread's first value column
+  const bool owns = jl < sh.columns && j0 < vdim;           // (threads that only fill the last wave own nothing)
+  const int k0 = ks * RS;
   const int inner = sh.heads * vdim;
   const int group = head / (sh.heads / sh.groups);
   const int b_col = inner + group * ns, c_col = inner + sh.groups * ns + group * ns;
-  float* S = MODE == 0 ? state + ((size_t)state_slots[req] * sh.heads + head) * ns * vdim
-                       : chunk_state + place * ns * vdim;
-  float s[SLICE];
+  // a head's state lies as [groups of four columns][ns rows][4]: a thread's rows are one run of 16-byte
+  // pieces, and the threads of a column group (neighbouring lanes) read neighbouring runs
+  const size_t head_elems = (size_t)((vdim + 3) / 4) * ns * 4;
+  float* S = (MODE == 0 ? state + ((size_t)state_slots[req] * sh.heads + head) * head_elems
+                        : chunk_state + place * head_elems) + ((size_t)(j0 >> 2) * ns + k0) * 4;
+  float s[RS][CS];
 #pragma unroll
-  for (int x = 0; x < SLICE; ++x) s[x] = (MODE != 1 && live && x < kn) ? S[(size_t)(k0 + x) * vdim + j] : 0.f;
+  for (int r = 0; r < RS; ++r) {
+    float4 row = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (MODE != 1 && owns && k0 + r < ns) row = *reinterpret_cast<const float4*>(S + r * 4);
+    s[r][0] = row.x; s[r][1] = row.y; s[r][2] = row.z; s[r][3] = row.w;
+  }
   const float rate = expf(a_log[head]), bias = dt_bias[head], d_skip = skip[head];
   float decayed = 1.f;      // the product of the chunk's decays (MODE 1)
 
   for (int t0 = first; t0 < end; t0 += TB) {
     const int tb = min(TB, end - t0);
-    for (int i = tid; i < tb * ns; i += nthreads) {
-      const int t = i / ns, n = i - t * ns;
+    for (int i = tid; i < tb * nsp; i += nthreads) {
+      const int t = i / nsp, n = i - t * nsp;
       const size_t row = (size_t)(t0 + t) * C;
-      // (every element forms its token's step size itself: the same float32 operations, one barrier less)
+      // (every element forms its token's step size itself: the same float32 operations, no barrier for it)
       const float dt = softplus(load_in<T>(dt_in, (size_t)(t0 + t) * ld + dt_col + head) + bias);
-      bb[t * nsp + n] = dt * Elem<T>::load(u + row + b_col + n);
-      cc[t * nsp + n] = Elem<T>::load(u + row + c_col + n);
+      bb[i] = n < ns ? dt * Elem<T>::load(u + row + b_col + n) : 0.f;
+      cc[i] = n < ns ? Elem<T>::load(u + row + c_col + n) : 0.f;
       if (n == 0) aa[t] = expf(-rate * dt);
     }
-    float xloc[TB];
+    float xloc[TB][CS];
 #pragma unroll
-    for (int t = 0; t < TB; ++t) xloc[t] = (t < tb && live) ? Elem<T>::load(u + (size_t)(t0 + t) * C + head * vdim + j) : 0.f;
+    for (int t = 0; t < TB; ++t) {
+#pragma unroll
+      for (int c = 0; c < CS; ++c)
+        xloc[t][c] = (t < tb && owns && j0 + c < vdim) ? Elem<T>::load(u + (size_t)(t0 + t) * C + head * vdim + j0 + c) : 0.f;
+    }
     __syncthreads();
+    float outs[TB * CS];      // this thread's share of the round's outputs: [token][column]
+#pragma unroll
+    for (int i = 0; i < TB * CS; ++i) outs[i] = 0.f;
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
       if (t < tb) {
-        const float xj = xloc[t], decay = aa[t];
-        float o = 0.f;
+        const float decay = aa[t];
+        float o[CS] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int x = 0; x < SLICE; x += 4) {
-          if (x < kn) {
-            const int at = t * nsp + k0 + x;        // (k0 and nsp are multiples of four)
-            const float4 b4 = *reinterpret_cast<const float4*>(bb + at);
-            const float4 c4 = *reinterpret_cast<const float4*>(cc + at);
-            const float bv[4] = {b4.x, b4.y, b4.z, b4.w}, cv[4] = {c4.x, c4.y, c4.z, c4.w};
+        for (int r0 = 0; r0 < RS; r0 += 4) {
+          const float4 b4 = *reinterpret_cast<const float4*>(bb + t * nsp + k0 + r0);
+          const float4 c4 = *reinterpret_cast<const float4*>(cc + t * nsp + k0 + r0);
+          const float bv[4] = {b4.x, b4.y, b4.z, b4.w}, cv[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (x + e < kn) {
-                s[x + e] = fmaf(decay, s[x + e], bv[e] * xj);
-                if (MODE != 1) o = fmaf(cv[e], s[x + e], o);
-              }
+          for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int c = 0; c < CS; ++c) {
+              s[r0 + e][c] = fmaf(decay, s[r0 + e][c], bv[e] * xloc[t][c]);
+              if (MODE != 1) o[c] = fmaf(cv[e], s[r0 + e][c], o[c]);
             }
           }
         }
-        if (MODE == 1) decayed *= decay;
-        else if (worker) part[(ks * TB + t) * CT + jl] = o;
-      }
-    }
-    __syncthreads();
-    if (MODE == 1) continue;     // (every thread alike; the barrier above keeps the staging of the next round off this one's reads)
-    for (int t = worker ? ks : tb; t < tb; t += KS) {
-      float o = 0.f;
-      for (int q = 0; q < KS; ++q) o += part[(q * TB + t) * CT + jl];
-      if (live) {
-        const size_t at = (size_t)(t0 + t) * inner + head * vdim + j;
-        y[at] = fmaf(d_skip, Elem<T>::load(u + (size_t)(t0 + t) * C + head * vdim + j), o);
-      }
-    }
-    __syncthreads();     // (the next round's staging writes what this round's sums have read)
-  }
-  if (MODE != 2 && live) {
+        if (MODE == 1) {
+          decayed *= decay;
+        } else {
 #pragma unroll
-    for (int x = 0; x < SLICE; ++x)
-      if (x < kn) S[(size_t)(k0 + x) * vdim + j] = s[x];
+          for (int c = 0; c < CS; ++c)      // (the skip term once a column group: in its first lane's share)
+            outs[t * CS + c] = ks == 0 ? fmaf(d_skip, xloc[t][c], o[c]) : o[c];
+        }
+      }
+    }
+    if (MODE != 1) {
+      // the sums over the KS lanes that share the column group (every lane of the wave takes part)
+      static_assert(TB * CS == 32, "sum_and_deal takes 32 values");
+      sum_and_deal<TB * CS, KS / 2>(outs, ks);
+      constexpr int LEFT = KS <= TB * CS ? TB * CS / KS : 1;           // sums a lane is left with
+      constexpr int SHARE = KS > TB * CS ? KS / (TB * CS) : 1;         // lanes that are left with the same sum
+      const int base = ks * LEFT / SHARE;
+      const bool writes = owns && (ks & (SHARE - 1)) == 0;
+#pragma unroll
+      for (int i = 0; i < LEFT; ++i) {
+        const int t = (base + i) / CS, c = (base + i) % CS;
+        if (writes && t < tb && j0 + c < vdim) y[(size_t)(t0 + t) * inner + head * vdim + j0 + c] = outs[i];
+      }
+    }
+    __syncthreads();     // (the next round's staging writes what this round has read)
+  }
+  if (MODE != 2 && owns) {
+#pragma unroll
+    for (int r = 0; r < RS; ++r)      // (columns behind vdim stay zeros: their x is zero)
+      if (k0 + r < ns) *reinterpret_cast<float4*>(S + r * 4) = make_float4(s[r][0], s[r][1], s[r][2], s[r][3]);
   }
   if (MODE == 1 && tid == 0 && blockIdx.z == 0) chunk_decay[place] = decayed;
 }
@@ -343,33 +396,48 @@ int launch_scan(const void* u, int C, SsmIn dt, long ld, int dt_col, const float
   sh.groups = groups;
   sh.ns = ns;
   sh.vdim = vdim;
-  sh.columns = splits > 1 ? (vdim + splits - 1) / splits : vdim;
-  const int most = max(1, min(16, 1024 / sh.columns));
-  sh.slice = max(4, ((ns + most - 1) / most + 3) / 4 * 4);
-  sh.slices = (ns + sh.slice - 1) / sh.slice;
-  if (sh.slice > 64) return -1;
-  const int threads = (sh.columns * sh.slices + kWave - 1) / kWave * kWave;
-  if (threads > 1024) return -1;
-  const int nsp = (ns + 3) & ~3;
-  const size_t lds = ((size_t)2 * kScanTokens * nsp + kScanTokens + (size_t)sh.slices * kScanTokens * sh.columns) * 4;
-  if (lds > 64 * 1024) return -1;
-  const dim3 grid(chunk > 0 ? R * max_chunks : R, heads, splits);
-#define TK_SSD_AS(SLICE, MODE)                                                                                \
-  ssd_scan_kernel<T, SLICE, MODE><<<grid, threads, lds, stream>>>((const T*)u, C, dt, ld, dt_col, dt_bias,    \
-                                                                 a_log, skip, state, q_start, state_slots, y, \
-                                                                 sh, chunk, max_chunks, chunk_state, chunk_decay)
-#define TK_SSD(MODE)                     \
-  {                                      \
-    if (sh.slice <= 4) TK_SSD_AS(4, MODE);        \
-    else if (sh.slice <= 16) TK_SSD_AS(16, MODE); \
-    else TK_SSD_AS(64, MODE);                     \
+  // rows a thread (4, or more where the state is long) and threads a column group (a power of two up to a wave)
+  const int rs = ns <= 256 ? 4 : ns <= 512 ? 8 : 16;
+  const int ks = ns <= 16 ? 4 : ns <= 64 ? 16 : ns <= 128 ? 32 : 64;
+  if (ns > 1024) return -1;
+  sh.slices = ks;
+  const int col_groups = (vdim + 3) / 4;
+  sh.columns = max(1, min((col_groups + splits - 1) / splits, 1024 / ks));
+  const int shares = (col_groups + sh.columns - 1) / sh.columns;
+  const int threads = (sh.columns * ks + kWave - 1) / kWave * kWave;
+  const size_t lds = ((size_t)2 * kScanTokens * ks * rs + kScanTokens) * 4;
+  const dim3 grid(chunk > 0 ? R * max_chunks : R, heads, shares);
+#define TK_SSD_AS(RS, KS, MODE)                                                                               \
+  {                                                                                                           \
+    if (lds > 48 * 1024) {                                                                                    \
+      static bool raised = false;                                                                             \
+      if (!raised) {                                                                                          \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&ssd_scan_kernel<T, RS, KS, MODE>),             \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024) != hipSuccess)         \
+          return -1;                                                                                          \
+        raised = true;                                                                                        \
+      }                                                                                                       \
+    }                                                                                                         \
+    ssd_scan_kernel<T, RS, KS, MODE><<<grid, threads, lds, stream>>>((const T*)u, C, dt, ld, dt_col, dt_bias, \
+                                                                    a_log, skip, state, q_start, state_slots, \
+                                                                    y, sh, chunk, max_chunks, chunk_state,    \
+                                                                    chunk_decay);                             \
+  }
+#define TK_SSD(MODE)                               \
+  {                                                \
+    if (rs == 16) TK_SSD_AS(16, 64, MODE)          \
+    else if (rs == 8) TK_SSD_AS(8, 64, MODE)       \
+    else if (ks == 64) TK_SSD_AS(4, 64, MODE)      \
+    else if (ks == 32) TK_SSD_AS(4, 32, MODE)      \
+    else if (ks == 16) TK_SSD_AS(4, 16, MODE)      \
+    else TK_SSD_AS(4, 4, MODE)                     \
   }
   if (chunk <= 0) {
     TK_SSD(0)
     return launch_status();
   }
   TK_SSD(1)
-  const int elems = ns * vdim;
+  const int elems = (vdim + 3) / 4 * ns * 4;
   ssd_chunk_starts_kernel<<<dim3(R, heads, (elems + 1023) / 1024), 256, 0, stream>>>(state, q_start, state_slots, chunk_state,
                                                                                    chunk_decay, heads, elems, chunk);
   TK_SSD(2)
@@ -406,10 +474,11 @@ TK_API int tk_conv_silu(int dtype, const void* proj, int in_f32, int parts, long
 }
 
 // u: [N, C] in dtype, C = heads * vdim + 2 * groups * ns ([x | B | C]).  dt: column dt_col .. + heads of rows
-// ld long (dtype, float32 or partial sums).  state float32 [slots, heads, ns, vdim].  y float32 [N, heads * vdim].
+// ld long (dtype, float32 or partial sums).  state float32 [slots, heads, ceil(vdim / 4), ns, 4] (a head's columns
+// in groups of four, the columns behind vdim zeros).  y float32 [N, heads * vdim].
 // splits: blocks that share a head's value columns.  chunk > 0: portions are cut into chunks of so many tokens
 // that run side by side; max_chunks: the most chunks a request of the step has; chunk_state float32
-// [chunks of the step, heads, ns, vdim] and chunk_decay float32 [chunks of the step, heads] are scratch.
+// [chunks of the step, heads, ceil(vdim / 4), ns, 4] and chunk_decay float32 [chunks of the step, heads] are scratch.
 TK_API int tk_ssd_scan(int dtype, const void* u, const void* dt, int dt_f32, int dt_parts, long dt_stride, long ld,
                        int dt_col, const float* dt_bias, const float* a_log, const float* skip, float* state,
                        const int* q_start, const int* state_slots, float* y, int R, int heads, int groups, int ns,

@@ -990,15 +990,16 @@ def ssd_scan(u: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Te
     """Per request and head over the step's tokens in order: dt = softplus(proj[t, dt_col + head] + dt_bias),
     S <- exp(-exp(a_log) dt) S + dt B_t x_t^T, y_t = S^T C_t + skip x_t, with x, B, C the columns of ``u``
     ([N, heads * vdim + 2 groups * state_size], the convolution's output; head h reads group h // (heads / groups)),
-    S float32 [slots, heads, state_size, vdim] (kept) and y float32 [N, heads * vdim]."""
+    y float32 [N, heads * vdim] and the state S float32 [slots, heads, ceil(vdim / 4), state_size, 4] (kept; a head's
+    value columns in groups of four, which is how the kernel's threads own them; columns behind vdim are zeros)."""
     _gpu(u, proj, dt_bias, a_log, skip, state, y)
     n = y.shape[0]
     c = heads * vdim + 2 * groups * state_size
     _need(heads % groups == 0 and u.shape == (n, c) and y.dtype == torch.float32 and y.shape == (n, heads * vdim),
           "the scan's operands do not match its sizes")
     _need(all(t.dtype == torch.float32 and t.numel() == heads for t in (dt_bias, a_log, skip)), "a head's constants are float32 [heads]")
-    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, state_size, vdim),
-          "the state is float32 [slots, heads, state, vdim]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, -(-vdim // 4), state_size, 4),
+          "the state is float32 [slots, heads, ceil(vdim / 4), state, 4]")
     _need(1 <= vdim <= 1024 and 1 <= state_size <= 1024 and batch.num_tokens == n, "the scan takes sizes up to 1,024")
     pointer, is_f32, parts, stride, ld = _ssm_in(proj, n, u.dtype, "projections")
     _need(0 <= dt_col and dt_col + heads <= ld, "the step sizes lie outside the projections")
@@ -1012,7 +1013,7 @@ def ssd_scan(u: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Te
         chunk = SSM_CHUNK_TOKENS
         max_chunks = -(-batch.max_q_len // chunk)
         blocks = n // chunk + batch.num_requests        # (no step has more chunks than this)
-        chunk_state = torch.empty((blocks, heads, state_size, vdim), dtype=torch.float32, device=y.device)
+        chunk_state = torch.empty((blocks, heads, -(-vdim // 4), state_size, 4), dtype=torch.float32, device=y.device)
         chunk_decay = torch.empty((blocks, heads), dtype=torch.float32, device=y.device)
     splits = ssd_column_splits(blocks, heads, vdim, batch.max_q_len)
     _note(f"{n}x{heads}x{state_size}x{vdim}", n * (c * u.element_size() + heads * vdim * 4), 6.0 * n * heads * state_size * vdim)

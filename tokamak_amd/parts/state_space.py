@@ -27,7 +27,8 @@ class SelectiveStateSpace(Mixer):
 
     y (heads side by side) is multiplied by silu(z), THEN divided by its root mean square over each
     of ``norm_groups`` equal parts of the row (``norm_eps``) and multiplied by a weight, and
-    projected by W_o.  The request's state is S (float32) and the convolution's last taps - 1 inputs,
+    projected by W_o.  The request's state is S (float32, held as [heads, value_dim / 4, N, 4]) and the
+    convolution's last taps - 1 inputs,
     both carried from step to step; step sizes, decays, the recurrence, the gate's product and the
     norm are float32.
     Tensors: in, conv, conv.b, dt_bias, A_log, D, norm, o behind the part's prefix.
@@ -81,7 +82,8 @@ class SelectiveStateSpace(Mixer):
         self.gain = fetch(prefix + norm)
 
     def state_request(self) -> dict[str, StateArray]:
-        out = {"S": StateArray((self.num_heads, self.state_size, self.value_dim), torch.float32)}
+        # (a head's value columns in groups of four, as the scan's threads own them)
+        out = {"S": StateArray((self.num_heads, -(-self.value_dim // 4), self.state_size, 4), torch.float32)}
         if self.conv_taps > 1:
             out["conv"] = StateArray((self.conv_taps - 1, self.conv_channels), torch.float32)
         return out
