@@ -254,7 +254,7 @@ def test_window_attention_with_kept_first_positions_alone(dtype, name):
     LDS, and for single tokens the heads-as-columns form; else the generic kernel."""
     a = ATTENTIONS[name]
     width = 64
-    page = 16 if a["dim"] * a["heads"] >= 96 else 8
+    page = 16 if a["dim"] * a["heads"] >= 64 else 8
     cfg = model_json([attention(**a, scale=3.0 * a["dim"] ** -0.5, mlp=None)], width=width)
     m = cfg["layers"][0]["mixer"]
     w = random_weights(cfg, seed=a["dim"] + a["heads"])
