@@ -144,7 +144,7 @@ SSMS = {
     "odd": dict(heads=3, vdim=20, state=24, groups=1, conv=3, norm_groups=5),
     "ones": dict(heads=2, vdim=8, state=5, groups=2, conv=1, norm_groups=1),
     "wide": dict(heads=6, vdim=64, state=128, groups=3, conv=8, norm_groups=6),
-    "taps2": dict(heads=8, vdim=32, state=48, groups=2, conv=2, norm_groups=16),
+    "taps2": dict(heads=8, vdim=24, state=40, groups=4, conv=2, norm_groups=16),
 }
 
 
@@ -216,7 +216,7 @@ def test_state_space_mixer_in_portions_over_state_slots(dtype, name):
 
 ATTENTIONS = {
     "g2": dict(heads=4, kv_heads=2, dim=16, vdim=16, rot=8, window=24, keep_first=3),
-    "g4-yarn": dict(heads=4, kv_heads=1, dim=96, vdim=96, rot=24, base=1e6, yarn=(8.0, 64.0, 32.0, 1.0), window=40, keep_first=6),
+    "g4-yarn": dict(heads=4, kv_heads=1, dim=80, vdim=48, rot=20, base=5e5, yarn=(4.0, 64.0, 16.0, 2.0), window=44, keep_first=5),
     "g1-long-keep": dict(heads=2, kv_heads=2, dim=40, vdim=16, rot=0, window=33, keep_first=70),
     "g8": dict(heads=16, kv_heads=2, dim=24, vdim=32, rot=24, window=30, keep_first=17),
     "g9-keep1": dict(heads=9, kv_heads=1, dim=32, vdim=32, rot=16, window=64, keep_first=1),
@@ -285,7 +285,7 @@ def test_window_attention_with_kept_first_positions_alone(dtype, name):
 
 LATENTS = {
     "base": dict(heads=2, dim=16, vdim=16, kv_rank=32, q_rank=24),
-    "mfma": dict(heads=4, dim=64, vdim=64, kv_rank=128, q_rank=80),
+    "mfma": dict(heads=8, dim=32, vdim=48, kv_rank=128, q_rank=72),
     "odd": dict(heads=3, dim=20, vdim=36, kv_rank=45, q_rank=17),
     "many": dict(heads=20, dim=8, vdim=16, kv_rank=64, q_rank=8),
     "one": dict(heads=1, dim=8, vdim=8, kv_rank=16, q_rank=1),
@@ -358,7 +358,7 @@ def test_dense_feed_forward_with_biases(dtype, rows, width, ff):
 
 ROUTERS = {
     "base": dict(n=8, top=2, ff=32, scale=1.5, groups=(4, 2), shared=24),
-    "given-like": dict(n=12, top=3, ff=24, scale=2.5, groups=(4, 3), shared=40),
+    "threes": dict(n=15, top=3, ff=24, scale=2.5, groups=(5, 3), shared=40),
     "ones": dict(n=6, top=1, ff=16, scale=None, groups=(6, 1), shared=None),
     "no-groups": dict(n=5, top=2, ff=40, scale=0.5, groups=None, shared=8),
     "all-kept": dict(n=9, top=4, ff=24, scale=1.0, groups=(3, 3), shared=None),
@@ -420,7 +420,7 @@ def test_grouped_router_and_experts_with_a_shared_one(dtype, name, correction):
 # -- whole models -------------------------------------------------------------------
 SHAPES = {
     "base": dict(cfg=model_json([latent(mlp=dense(40)), mamba(), attention(), latent(kv_from=0), mamba(mlp=dense(24)),
-                                 attention(heads=8, kv_heads=1, window=40, keep_first=6)]), page=16),
+                                 attention(heads=8, kv_heads=1, window=36, keep_first=5)]), page=16),
     "odd": dict(cfg=model_json([mamba(heads=3, vdim=20, state=24, groups=1, conv=3, norm_groups=5, mlp=experts(5, 1, 24, None, None, None)),
                                 attention(heads=3, kv_heads=3, dim=20, vdim=40, rot=12, yarn=(2.0, 16.0, 4.0, 1.0), window=19, keep_first=0, mlp=None),
                                 latent(heads=3, dim=20, vdim=36, kv_rank=45, q_rank=17, mlp=experts(6, 2, 40, 0.7, (3, 2), 16)),

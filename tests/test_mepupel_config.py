@@ -12,7 +12,7 @@ from mepupel_util import (attention, dense, double, experts, latent, mamba, mode
                           tokens, write_folder)
 
 CFG = model_json([latent(mlp=dense(40)), mamba(), attention(), latent(kv_from=0), mamba(mlp=None),
-                  attention(rot=16, yarn=(8.0, 64.0, 32.0, 1.0), window=40, keep_first=6)])
+                  attention(rot=16, yarn=(4.0, 64.0, 16.0, 2.0), window=44, keep_first=5)])
 
 
 def test_a_folder_is_found_by_its_architecture_key_and_round_trips(tmp_path):
@@ -40,7 +40,7 @@ def test_run_order_and_cache_slots_of_borrowed_latents():
         assert ("feed_forward_norm" in roles) == (layer["mlp"] is not None) == ("feed_forward" in roles)
         assert spec.block.kind == "parallel_sublayers" and spec.block["branch_scale"] == 0.5
     assert "position" in dict(made.layers[2].parts) and "position" not in dict(made.layers[0].parts)
-    assert made.layers[5].role("position").spec["yarn"] == (8.0, 64.0, 32.0, 1.0)
+    assert made.layers[5].role("position").spec["yarn"] == (4.0, 64.0, 16.0, 2.0)
 
 
 def test_tensor_names_and_shapes_match_a_list_written_independently():
@@ -186,7 +186,7 @@ def test_plain_rotation_pairs_halves_and_stretches_slow_frequencies():
     assert all(a >= b - 1e-12 for a, b in zip(ratios, ratios[1:]))
 
 
-@pytest.mark.parametrize("rot", [dict(base=10000.0, dims=16), dict(base=1e6, dims=24, scaling=dict(factor=8.0, original=1024, fast=32.0, slow=1.0)),
+@pytest.mark.parametrize("rot", [dict(base=10000.0, dims=16), dict(base=2e5, dims=20, scaling=dict(factor=6.0, original=512, fast=16.0, slow=2.0)),
                                  dict(base=500.0, dims=8, scaling=dict(factor=8.0, original=16, fast=4.0, slow=0.5))])
 def test_the_engines_frequencies_match_the_plain_ones(rot):
     from tokamak_amd.parts.rotary import yarn_frequencies
