@@ -642,3 +642,30 @@ def test_trace_runner_and_command_line(models, tmp_path):
     done = subprocess.run([sys.executable, "-m", "tokamak_amd.cli", "--random-weights", "mepupel-tiny", "--prompt-ids",
                            "1,2,3", "--max-new-tokens", "3", "--quiet"], cwd=ROOT, capture_output=True, text=True, timeout=240)
     assert done.returncode == 0, done.stderr[-2000:]
+
+
+def test_layers_of_a_real_width(tmp_path):
+    """Six layers of the 0.6B-class preset (state-space heads of 64 with a state of 128, attention heads of 128,
+    a latent of 256 under 16 heads, 16 experts) with a small vocabulary: the library products of long
+    portions, the tuned attention kernels, the scan in chunks, the experts grouped on the matrix cores.
+    float32 row by row in every cutting; bfloat16 by its median (its routers meet close calls)."""
+    import dataclasses
+
+    from tokamak_amd.config.registry import find_preset
+    from tokamak_amd.engine.runner import ModelRunner
+
+    arch, full = find_preset("mepupel-0.6b")
+    cfg = arch.to_json(dataclasses.replace(arch.shorten(full, 6), vocab_size=512))
+    w = random_weights(cfg, 5)
+    folder = write_folder(tmp_path / "wide", cfg, w)
+    toks = tokens(512, 200, 3)
+    expected = {"x": oracle_logits(cfg, w, toks)}
+    cuts = [whole({"x": toks}), tail_one_by_one("x", toks, tail=50), portions("x", toks, sizes=(70, 2, 65, 13, 50))]
+    runner = ModelRunner.from_folder(folder, dtype="float32", page_size=16, kv_pool_tokens=512, max_requests=2)
+    for steps in cuts:
+        check_rows(steps, run_steps(runner, steps), expected, "float32")
+    del runner
+    runner = ModelRunner.from_folder(folder, dtype="bfloat16", page_size=16, kv_pool_tokens=512, max_requests=2)
+    for steps in cuts:
+        errors = [e for e, _ in row_errors(steps, run_steps(runner, steps), expected)]
+        assert np.median(errors) < 0.03, np.median(errors)
